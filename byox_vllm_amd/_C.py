@@ -14,7 +14,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 # NV_HIP_LIB points at another build of the same library (A/B measurements); the default is the in-tree build.
 LIB_PATH = os.environ.get("NV_HIP_LIB") or os.path.join(_HERE, "libnv_hip.so")
 
-NV_BF16, NV_F16 = 0, 1
+NV_BF16, NV_F16, NV_F32 = 0, 1, 2
 W_DENSE, W_INT8, W_INT4, W_DENSE_TILED = 0, 1, 2, 3
 GEMM_SILU_MUL, GEMM_PARTIAL_OUT = 1, 2
 
@@ -65,6 +65,18 @@ _PROTOS = {
     "nv_stage_decode_packed": (_i, [_p, _i, _i, _i, _p, _p, _p, _p, _p, _i, _p, _p, _p]),
     "nv_stage_decode_packed_advance": (_i, [_p, _i, _p, _p, _p, _p, _p, _i, _p, _p, _p, _i, _p]),
     "nv_stage_decode_inputs": (_i, [_p, _p, _p, _p, _p, _i, _p, _p, _p, _p, _p, _i, _i, _i, _p]),
+    "nv_linear": (_i, [_p, _i64, _p, _p, _i64, _p, _p, _i64, _i, _i64, _i, _i, _i, _i64, _i64, _i64, _i64, _p, _i, _i, _p,
+                       _i64, _f, _i, _p]),
+    "nv_embed_scale": (_i, [_p, _p, _p, _i64, _i, _i64, _f, _i, _p]),
+    "nv_dyt_norm": (_i, [_p, _p, _i64, _p, _p, _p, _p, _p, _i64, _i, _i, _p]),
+    "nv_rmsnorm_f32": (_i, [_p, _i64, _p, _p, _i64, _i64, _i, _f, _i, _p]),
+    "nv_gla_recurrent": (_i, [_p, _i64, _i, _i, _i, _i, _p, _i64, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _f, _f, _f, _i, _p]),
+    "nv_latent_kv_store": (_i, [_p, _i64, _p, _p, _p, _f, _p, _p, _i64, _i, _i, _i, _f, _i, _p]),
+    "nv_latent_q_rope": (_i, [_p, _i64, _p, _p, _f, _p, _i64, _i, _i, _i, _i, _i, _i, _p]),
+    "nv_latent_attn": (_i, [_p, _p, _p, _i, _p, _p, _p, _p, _i64, _i, _i, _i, _i, _i, _f, _i, _p]),
+    "nv_moe_route": (_i, [_p, _i64, _p, _p, _i64, _i, _i, _p]),
+    "nv_moe_sort": (_i, [_p, _i64, _i, _i, _p, _p, _p, _p]),
+    "nv_moe_combine": (_i, [_p, _p, _p, _i, _p, _p, _i64, _p, _i64, _i, _p]),
 }
 
 _lib = None
@@ -84,10 +96,20 @@ def lib():
                 "(hipcc --offload-arch=gfx950). There is no CPU fallback for the HIP path.")
         handle = C.CDLL(LIB_PATH)
         for name, (res, args) in _PROTOS.items():
-            fn = getattr(handle, name)
+            fn = getattr(handle, name, None)
+            if fn is None:       # a library linked from the sources of one model only (byox_vllm_amd.build.ensure)
+                setattr(handle, name, _absent(name))
+                continue
             fn.restype, fn.argtypes = res, args
         _lib = handle
     return _lib
+
+
+def _absent(name: str):
+    def call(*_):
+        raise RuntimeError(f"{LIB_PATH} was linked without {name}: build the whole library with "
+                           "`python -c 'import __graft_entry__ as g; g.build()'`")
+    return call
 
 
 def check(code: int, what: str) -> None:
@@ -95,11 +117,13 @@ def check(code: int, what: str) -> None:
         raise RuntimeError(f"{what} failed ({code}): {lib().nv_last_error().decode()}")
 
 
-def dtype_code(dt: torch.dtype) -> int:
+def dtype_code(dt: torch.dtype, allow_f32: bool = False) -> int:
     if dt == torch.bfloat16:
         return NV_BF16
     if dt == torch.float16:
         return NV_F16
+    if dt == torch.float32 and allow_f32:     # only the entry points that take NV_F32 pass allow_f32
+        return NV_F32
     raise TypeError(f"the HIP path computes in bf16 or fp16, got {dt}")
 
 

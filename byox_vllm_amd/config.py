@@ -28,6 +28,10 @@ def _load_hf_config(path: str):
 
     with open(os.path.join(path, "config.json")) as f:
         raw = json.load(f)
+    from byox_vllm_amd.models.registry import read_config
+    own = read_config(raw, path)      # a registered model class may read its own configuration format
+    if own is not None:
+        return own
     rope = raw.get("rope_parameters") or {}
     rope_theta = raw.get("rope_theta", rope.get("rope_theta", 1000000))
     rope_scaling = raw.get("rope_scaling")
@@ -64,6 +68,8 @@ class Config:
     state_dict: Any = None   # optional in-memory checkpoint keyed by the packed parameter names
     tp_port: int = 0         # rendezvous port of this engine's tensor-parallel ranks (0: LLMEngine picks a free one)
     shm_name: str = ""       # name of this engine's control-message shared memory ("": LLMEngine derives a unique one)
+    dtype: Any = None        # compute/storage dtype override (torch dtype or its name); None: what the checkpoint says
+    num_state_slots: int = 0  # models with a recurrent state: requests that can be live at once (0: max_num_seqs)
 
     def __post_init__(self):
         assert self.kvcache_block_size % 16 == 0 and self.kvcache_block_size > 0
@@ -74,8 +80,15 @@ class Config:
             self.hf_config = _load_hf_config(self.model)
             if self.quantization is None:       # a checkpoint written by utils/quantize.py names its format
                 self.quantization = getattr(self.hf_config, "quantization", None)
+        if self.dtype is not None:
+            self.hf_config.dtype = getattr(torch, self.dtype) if isinstance(self.dtype, str) else self.dtype
         if getattr(self.hf_config, "dtype", None) is None:
             self.hf_config.dtype = torch.bfloat16
+        from byox_vllm_amd.models.registry import model_class
+        # models that step through prompt pieces and decoded tokens in one batch (Scheduler.schedule_portions)
+        self.portioned = bool(getattr(model_class(self.hf_config), "portioned", False))
+        if self.portioned and self.num_state_slots <= 0:
+            self.num_state_slots = self.max_num_seqs
         self.max_model_len = min(self.max_model_len, self.hf_config.max_position_embeddings)
         assert self.max_num_batched_tokens >= self.max_model_len
 

@@ -1,0 +1,193 @@
+// nv_linear: out = epilogue(A W^T + bias) for any shape, in bf16 or true fp32 storage, fp32 accumulation on the matrix
+// cores (v_mfma_f32_16x16x32_bf16 / v_mfma_f32_16x16x4_f32).  One entry point covers the shapes the tiled decode GEMM
+// (nv_gemm) does not take: K or N that are no multiples of its tiles, fp32 models, batched products with one weight
+// per head, grouped products with one weight per expert over gathered rows, and the gated epilogues.
+//
+// A workgroup owns a 64 x 64 tile of the output: wavefront w the 16 columns n0 + 16 w .. and all four 16-row
+// sub-tiles.  Operands go from memory straight into MFMA fragments (both are K-contiguous rows, which is the fragment
+// layout: lane (c, g) holds row c, k = k0 + 8 g .. + 8), so there is no LDS stage; the 4 wavefronts re-read the A rows
+// through the L1.  D[n][m] is accumulated (the weight fragment is the first operand), which leaves every lane with
+// four consecutive output columns.
+#include "anyt.h"
+
+namespace {
+
+struct LinArgs {
+  const void* a;
+  int64_t a_rs;
+  const int32_t* a_rows;
+  const void* w;
+  int64_t w_rs;
+  const void* bias;
+  void* out;
+  int64_t out_rs;
+  int64_t M;
+  int N, K;
+  int64_t a_bs, w_bs, out_bs, bias_bs;
+  const int32_t* group_off;
+  const float* epi_ptr;
+  int64_t epi_rs;
+  float epi_c;
+  int act;
+  int vec_a, vec_w;
+};
+
+enum { EPI_NONE = 0, EPI_GLU = 1, EPI_SOFTCAP = 2, EPI_ROW_GATE = 3 };
+
+template <typename T> struct Frag;
+template <> struct Frag<bf16_t> {
+  typedef bf16x8 type;
+  static constexpr int KS = 32, PER = 8;
+};
+template <> struct Frag<float> {
+  typedef f32x4 type;
+  static constexpr int KS = 16, PER = 4;
+};
+
+template <typename T>
+__device__ __forceinline__ typename Frag<T>::type load_frag(const T* row, int k, int K, bool vec) {
+  typedef typename Frag<T>::type F;
+  F r;
+  if (row == nullptr) {
+#pragma unroll
+    for (int e = 0; e < Frag<T>::PER; ++e) r[e] = (T)0.0f;
+    return r;
+  }
+  if (vec && k + Frag<T>::PER <= K) return *reinterpret_cast<const F*>(row + k);
+#pragma unroll
+  for (int e = 0; e < Frag<T>::PER; ++e) r[e] = (k + e < K) ? row[k + e] : (T)0.0f;
+  return r;
+}
+
+__device__ __forceinline__ f32x4 mma(bf16x8 a, bf16x8 b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+__device__ __forceinline__ f32x4 mma(f32x4 a, f32x4 b, f32x4 c) {
+  // lane group g supplies k = k0 + 4 g + e in step e: over the four steps the sixteen k of the block are each used once
+#pragma unroll
+  for (int e = 0; e < 4; ++e) c = __builtin_amdgcn_mfma_f32_16x16x4f32(a[e], b[e], c, 0, 0, 0);
+  return c;
+}
+
+template <typename T, typename TO, int EPI>
+__global__ __launch_bounds__(256) void linear_kernel(LinArgs p) {
+  typedef typename Frag<T>::type F;
+  constexpr int KS = Frag<T>::KS, PER = Frag<T>::PER;
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int c = lane & 15, g = lane >> 4;
+  const int z = blockIdx.z;
+  int64_t lo = 0, hi = p.M;
+  if (p.group_off) {
+    lo = p.group_off[z];
+    hi = p.group_off[z + 1];
+  }
+  const int64_t mbase = lo + (int64_t)blockIdx.y * 64;
+  if (mbase >= hi) return;
+  const int nsub = (int)((hi - mbase + 15) / 16 < 4 ? (hi - mbase + 15) / 16 : 4);
+  const int n0 = blockIdx.x * 64 + wv * 16;
+  if (n0 >= p.N) return;
+
+  const T* A = reinterpret_cast<const T*>(p.a) + z * p.a_bs;
+  const T* W = reinterpret_cast<const T*>(p.w) + z * p.w_bs;
+  const T* wrow = (n0 + c < p.N) ? W + (int64_t)(n0 + c) * p.w_rs : nullptr;
+  const T* urow = nullptr;
+  if constexpr (EPI == EPI_GLU) urow = (n0 + c < p.N) ? W + (int64_t)(p.N + n0 + c) * p.w_rs : nullptr;
+  const T* arow[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int64_t s = mbase + 16 * i + c;
+    arow[i] = nullptr;
+    if (s < hi) arow[i] = A + (int64_t)(p.a_rows ? p.a_rows[s] : s) * p.a_rs;
+  }
+  f32x4 acc[4], accu[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) acc[i] = accu[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  for (int k0 = 0; k0 < p.K; k0 += KS) {
+    const int k = k0 + PER * g;
+    const F wf = load_frag<T>(wrow, k, p.K, p.vec_w);
+    F uf;
+    if constexpr (EPI == EPI_GLU) uf = load_frag<T>(urow, k, p.K, p.vec_w);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if (i < nsub) {
+        const F xf = load_frag<T>(arow[i], k, p.K, p.vec_a);
+        acc[i] = mma(wf, xf, acc[i]);
+        if constexpr (EPI == EPI_GLU) accu[i] = mma(uf, xf, accu[i]);
+      }
+    }
+  }
+
+  TO* O = reinterpret_cast<TO*>(p.out) + z * p.out_bs;
+  const T* bias = p.bias ? reinterpret_cast<const T*>(p.bias) + z * p.bias_bs : nullptr;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int64_t s = mbase + 16 * i + c;
+    if (i >= nsub || s >= hi) continue;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int n = n0 + 4 * g + r;
+      if (n >= p.N) continue;
+      float v = acc[i][r];
+      if (bias) v += ld_f32<T>(bias + n);
+      if constexpr (EPI == EPI_GLU) {
+        const float u = accu[i][r];
+        v = (p.act == 1 ? gelu_tanh_f32(v) : silu_f32(v)) * u;
+      } else if constexpr (EPI == EPI_SOFTCAP) {
+        v = p.epi_c * tanhf(v / p.epi_c);
+      } else if constexpr (EPI == EPI_ROW_GATE) {
+        v *= sigmoid_f32(p.epi_ptr[s * p.epi_rs + z]);
+      }
+      st_f32<TO>(O + s * p.out_rs + n, v);
+    }
+  }
+}
+
+template <typename T, typename TO>
+int launch_epi(const LinArgs& p, int epi, dim3 grid, hipStream_t s) {
+  switch (epi) {
+    case EPI_NONE: linear_kernel<T, TO, EPI_NONE><<<grid, dim3(256), 0, s>>>(p); break;
+    case EPI_GLU: linear_kernel<T, TO, EPI_GLU><<<grid, dim3(256), 0, s>>>(p); break;
+    case EPI_SOFTCAP: linear_kernel<T, TO, EPI_SOFTCAP><<<grid, dim3(256), 0, s>>>(p); break;
+    default: linear_kernel<T, TO, EPI_ROW_GATE><<<grid, dim3(256), 0, s>>>(p); break;
+  }
+  return 0;
+}
+
+}  // namespace
+
+extern "C" int nv_linear(const void* a, int64_t a_row_stride, const int32_t* a_rows, const void* w, int64_t w_row_stride,
+                         const void* bias, void* out, int64_t out_row_stride, int out_dtype, int64_t M, int N, int K,
+                         int batch, int64_t a_batch_stride, int64_t w_batch_stride, int64_t out_batch_stride,
+                         int64_t bias_batch_stride, const int32_t* group_offsets, int epilogue, int act,
+                         const float* epi_ptr, int64_t epi_row_stride, float epi_const, int dtype, nv_stream_t stream) {
+  NV_CHECK_ARG(a && w && out, "nv_linear: null pointer");
+  NV_CHECK_ARG(dtype == NV_BF16 || dtype == NV_F32, "nv_linear: dtype %d is neither bf16 nor fp32", dtype);
+  NV_CHECK_ARG(out_dtype == NV_BF16 || out_dtype == NV_F32, "nv_linear: bad output dtype %d", out_dtype);
+  NV_CHECK_ARG(M >= 0 && N > 0 && K > 0 && batch > 0 && batch <= 65535, "nv_linear: bad shape M=%lld N=%d K=%d batch=%d",
+               (long long)M, N, K, batch);
+  NV_CHECK_ARG(epilogue >= EPI_NONE && epilogue <= EPI_ROW_GATE, "nv_linear: bad epilogue %d", epilogue);
+  NV_CHECK_ARG(epilogue != EPI_ROW_GATE || epi_ptr, "nv_linear: the row-gate epilogue needs its gate rows");
+  NV_CHECK_ARG(epilogue != EPI_SOFTCAP || epi_const > 0.0f, "nv_linear: the soft cap must be positive");
+  if (M == 0) return NV_OK;
+  const int64_t mtiles = (M + 63) / 64;
+  NV_CHECK_ARG(mtiles <= 65535, "nv_linear: %lld rows exceed one launch", (long long)M);
+  const size_t esz = dtype == NV_BF16 ? 2 : 4;
+  const int per = dtype == NV_BF16 ? 8 : 4;
+  LinArgs p{a, a_row_stride, a_rows, w, w_row_stride, bias, out, out_row_stride, M, N, K, a_batch_stride,
+            w_batch_stride, out_batch_stride, bias_batch_stride, group_offsets, epi_ptr, epi_row_stride, epi_const, act,
+            0, 0};
+  p.vec_a = (uintptr_t)a % 16 == 0 && a_row_stride % per == 0 && (a_batch_stride * esz) % 16 == 0;
+  p.vec_w = (uintptr_t)w % 16 == 0 && w_row_stride % per == 0 && (w_batch_stride * esz) % 16 == 0;
+  dim3 grid((unsigned)((N + 63) / 64), (unsigned)mtiles, (unsigned)batch);
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == NV_BF16) {
+    if (out_dtype == NV_BF16) launch_epi<bf16_t, bf16_t>(p, epilogue, grid, s);
+    else launch_epi<bf16_t, float>(p, epilogue, grid, s);
+  } else {
+    if (out_dtype == NV_BF16) launch_epi<float, bf16_t>(p, epilogue, grid, s);
+    else launch_epi<float, float>(p, epilogue, grid, s);
+  }
+  NV_CHECK_LAUNCH();
+  return NV_OK;
+}

@@ -1,0 +1,91 @@
+// Row-wise kernels of models whose residual stream lives in fp32: scaled embedding gather, Dynamic Tanh (an
+// element-wise norm with no statistics) fused with the residual add, and RMSNorm of fp32 rows.  Parameters are in the
+// model's storage type (bf16 or fp32), arithmetic is fp32, outputs round once to the storage type.
+#include "anyt.h"
+
+namespace {
+
+template <typename T>
+__global__ __launch_bounds__(256) void embed_scale_kernel(const int64_t* __restrict__ ids, const T* __restrict__ table,
+                                                          float* __restrict__ out, int width, int64_t vocab,
+                                                          float scale) {
+  const int64_t t = blockIdx.x;
+  int64_t id = ids[t];
+  if (id < 0 || id >= vocab) id = 0;
+  const T* row = table + id * width;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) out[t * width + i] = ld_f32<T>(row + i) * scale;
+}
+
+// x[r] += delta[r] (when delta is given; written back), out[i] = tanh(alpha * x[r]) * w + b with r = rows_idx ? rows_idx[i] : i
+template <typename T>
+__global__ __launch_bounds__(256) void dyt_kernel(float* __restrict__ x, const float* __restrict__ delta,
+                                                  int64_t delta_rs, const int32_t* __restrict__ rows_idx,
+                                                  const float* __restrict__ alpha, const T* __restrict__ w,
+                                                  const T* __restrict__ b, T* __restrict__ out, int n) {
+  const int64_t i = blockIdx.x;
+  const int64_t r = rows_idx ? rows_idx[i] : i;
+  const float a = alpha[0];
+  float* xr = x + r * n;
+  for (int j = threadIdx.x; j < n; j += blockDim.x) {
+    float v = xr[j];
+    if (delta) {
+      v += delta[r * delta_rs + j];
+      xr[j] = v;
+    }
+    st_f32<T>(out + i * n + j, tanhf(a * v) * ld_f32<T>(w + j) + ld_f32<T>(b + j));
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void rmsnorm_f32_kernel(const float* __restrict__ x, int64_t x_rs,
+                                                          const T* __restrict__ w, T* __restrict__ out, int64_t out_rs,
+                                                          int n, float eps) {
+  __shared__ float red[32];
+  const int64_t r = blockIdx.x;
+  const float* xr = x + r * x_rs;
+  float ss = 0.0f;
+  for (int j = threadIdx.x; j < n; j += blockDim.x) ss += xr[j] * xr[j];
+  ss = block_sum(ss, red);
+  const float inv = 1.0f / sqrtf(ss / (float)n + eps);
+  for (int j = threadIdx.x; j < n; j += blockDim.x) st_f32<T>(out + r * out_rs + j, xr[j] * inv * ld_f32<T>(w + j));
+}
+
+}  // namespace
+
+extern "C" int nv_embed_scale(const int64_t* ids, const void* table, float* out, int64_t tokens, int width, int64_t vocab,
+                              float scale, int dtype, nv_stream_t stream) {
+  NV_CHECK_ARG(ids && table && out, "nv_embed_scale: null pointer");
+  NV_CHECK_ARG(dtype == NV_BF16 || dtype == NV_F32, "nv_embed_scale: bad dtype %d", dtype);
+  NV_CHECK_ARG(tokens >= 0 && width > 0 && vocab > 0, "nv_embed_scale: bad shape");
+  if (tokens == 0) return NV_OK;
+  NV_DISPATCH_T(dtype, embed_scale_kernel<T><<<dim3((unsigned)tokens), dim3(256), 0, (hipStream_t)stream>>>(
+                           ids, (const T*)table, out, width, vocab, scale));
+  NV_CHECK_LAUNCH();
+  return NV_OK;
+}
+
+extern "C" int nv_dyt_norm(float* x, const float* delta, int64_t delta_row_stride, const int32_t* rows_idx,
+                           const float* alpha, const void* w, const void* b, void* out, int64_t rows, int n, int dtype,
+                           nv_stream_t stream) {
+  NV_CHECK_ARG(x && alpha && w && b && out, "nv_dyt_norm: null pointer");
+  NV_CHECK_ARG(dtype == NV_BF16 || dtype == NV_F32, "nv_dyt_norm: bad dtype %d", dtype);
+  NV_CHECK_ARG(!(delta && rows_idx), "nv_dyt_norm: the residual add and the row gather exclude each other");
+  NV_CHECK_ARG(rows >= 0 && n > 0, "nv_dyt_norm: bad shape");
+  if (rows == 0) return NV_OK;
+  NV_DISPATCH_T(dtype, dyt_kernel<T><<<dim3((unsigned)rows), dim3(256), 0, (hipStream_t)stream>>>(
+                           x, delta, delta_row_stride, rows_idx, alpha, (const T*)w, (const T*)b, (T*)out, n));
+  NV_CHECK_LAUNCH();
+  return NV_OK;
+}
+
+extern "C" int nv_rmsnorm_f32(const float* x, int64_t x_row_stride, const void* w, void* out, int64_t out_row_stride,
+                              int64_t rows, int n, float eps, int dtype, nv_stream_t stream) {
+  NV_CHECK_ARG(x && w && out, "nv_rmsnorm_f32: null pointer");
+  NV_CHECK_ARG(dtype == NV_BF16 || dtype == NV_F32, "nv_rmsnorm_f32: bad dtype %d", dtype);
+  NV_CHECK_ARG(rows >= 0 && n > 0, "nv_rmsnorm_f32: bad shape");
+  if (rows == 0) return NV_OK;
+  NV_DISPATCH_T(dtype, rmsnorm_f32_kernel<T><<<dim3((unsigned)rows), dim3(256), 0, (hipStream_t)stream>>>(
+                           x, x_row_stride, (const T*)w, (T*)out, out_row_stride, n, eps));
+  NV_CHECK_LAUNCH();
+  return NV_OK;
+}

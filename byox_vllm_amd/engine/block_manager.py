@@ -112,8 +112,25 @@ class BlockManager:
             if block.ref_count == 0:
                 self._release(block)
         seq.num_cached_tokens = 0
+        seq.num_computed_tokens = 0
         seq.block_table.clear()
         Sequence.table_epoch += 1
+
+    # -- portioned stepping ---------------------------------------------------
+    def blocks_short(self, seq: Sequence, num_tokens: int) -> int:
+        """Blocks ``seq`` still lacks to hold ``num_tokens`` tokens."""
+        return max(0, -(-num_tokens // self.block_size) - len(seq.block_table))
+
+    def extend(self, seq: Sequence, num_tokens: int) -> None:
+        """Grow the table of ``seq`` to cover ``num_tokens`` tokens, page by page as a prompt is stepped through in
+        portions.  No prefix hashes: this path serves models whose requests also carry state that pages cannot restore."""
+        short = self.blocks_short(seq, num_tokens)
+        if short > len(self.free_block_ids):
+            raise RuntimeError(f"{seq}: {short} more blocks needed, {len(self.free_block_ids)} free")
+        if short:
+            Sequence.table_epoch += 1
+        for _ in range(short):
+            seq.block_table.append(self._take(self.blocks[self.free_block_ids[0]]).block_id)
 
     # -- decode ---------------------------------------------------------------
     def can_append(self, seq: Sequence) -> bool:
@@ -139,3 +156,27 @@ class BlockManager:
             self.hash_to_block_id[h] = last.block_id
         else:
             assert last.hash == -1
+
+
+class StateSlotManager:
+    """Slots of the per-request recurrent state pools (one row per slot in every state-carrying layer's pool).  A slot
+    is handed out when a request is admitted and taken back when it ends or is preempted; its contents are not
+    cleared: a request that has no tokens behind it starts from zero inside the kernels."""
+
+    def __init__(self, num_slots: int):
+        self.num_slots = num_slots
+        self.free: deque[int] = deque(range(num_slots))
+
+    def can_allocate(self) -> bool:
+        return bool(self.free)
+
+    def allocate(self, seq: Sequence) -> None:
+        assert seq.state_slot < 0
+        if not self.free:
+            raise RuntimeError(f"{seq}: no free state slot ({self.num_slots} in use)")
+        seq.state_slot = self.free.popleft()
+
+    def release(self, seq: Sequence) -> None:
+        if seq.state_slot >= 0:
+            self.free.append(seq.state_slot)
+            seq.state_slot = -1

@@ -70,6 +70,15 @@ class LLMEngine:
         self.scheduler.add(Sequence(prompt, self.scheduler.block_manager.block_size, sampling_params))
 
     def _step(self):
+        if self.scheduler.portioned:
+            plan = self.scheduler.schedule_portions()
+            if not plan:
+                return [], 0
+            token_ids = self.model_runner.call("run_portions", plan)
+            prompt_tokens = sum(count for _, count in plan if count > 1)
+            finished = self.scheduler.advance(plan, token_ids)
+            outputs = [(seq.seq_id, seq.completion_token_ids) for seq in finished]
+            return outputs, (sum(count for _, count in plan) if prompt_tokens else -len(plan))
         seqs, is_prefill = self.scheduler.schedule()
         if not seqs:
             return [], 0

@@ -20,7 +20,7 @@ import torch.distributed as dist
 from byox_vllm_amd import kernels
 from byox_vllm_amd.engine.sequence import Sequence
 from byox_vllm_amd.layers.sampler import Sampler
-from byox_vllm_amd.models.qwen3 import Qwen3ForCausalLM
+from byox_vllm_amd.models.registry import model_class
 from byox_vllm_amd.utils.context import get_context, reset_context, set_context
 from byox_vllm_amd.utils.loader import init_random_weights, load_model
 from byox_vllm_amd.utils.logging import logger
@@ -102,16 +102,23 @@ class ModelRunner:
                 self.comm.connect(getattr(config, "tp_group", None))
                 set_comm(self.comm)
                 logger.info("tensor-parallel all-reduce over peer-mapped %s device memory", self.comm.memory_kind)
-            self.model = Qwen3ForCausalLM(hf_config)
+            self.model = model_class(hf_config)(hf_config)
+            self.portioned = bool(getattr(self.model, "portioned", False))
             self._load_weights()
             self.model.finalize(config.quantization)
             self.decode_result_policy = self._pick_decode_result_policy()
             self.prefill_result_policy = int(os.environ.get("NV_RESULT_POLICY_PREFILL", "0"))
             self.sampler = Sampler(seed=config.seed)
-            self._warmup_model()
-            self._allocate_kv_cache()
-            if not self.enforce_eager:
-                self._capture_graphs()
+            if self.portioned:
+                # models that step through run_portions: pages and state slots from the layers' own specs, eager steps
+                assert self.world_size == 1, "portioned models run on one rank"
+                self.enforce_eager = True
+                self._allocate_pools()
+            else:
+                self._warmup_model()
+                self._allocate_kv_cache()
+                if not self.enforce_eager:
+                    self._capture_graphs()
         except BaseException:
             self._release_after_failed_init()
             raise
@@ -511,6 +518,80 @@ class ModelRunner:
                 raise RuntimeError(f"rank {self.rank}: the peer-memory all-reduce timed out waiting for a peer "
                                    f"(nv_comm_error = {code}: phase {code - 1}); this step's hidden states are invalid")
 
+    # ------------------------------------------------------------------ portioned steps
+    def _allocate_pools(self) -> None:
+        """Cache memory of a portioned model: every layer that owns cache rows gets [blocks * block_size, width] in the
+        model dtype (one block table per request indexes all of them), every layer that owns a recurrent state gets
+        fp32 [slots, *shape].  Layers that read another layer's rows hold a reference to that layer."""
+        config, dtype = self.config, self.config.hf_config.dtype
+        pages, states = self.model.page_layers(), self.model.state_layers()
+        slots = max(1, config.num_state_slots or config.max_num_seqs)
+        state_bytes = sum(4 * slots * int(np.prod(m.state_spec()["shape"])) for m in states)
+        block_bytes = sum(m.page_spec()["width"] for m in pages) * self.block_size * dtype.itemsize
+        if config.num_kvcache_blocks <= 0:
+            free, total = torch.cuda.mem_get_info()
+            room = int(total * config.gpu_memory_utilization - (total - free)) - state_bytes
+            config.num_kvcache_blocks = max(1, room // max(block_bytes, 1)) if pages else 1
+        assert config.num_kvcache_blocks > 0
+        rows = config.num_kvcache_blocks * self.block_size
+        for m in pages:
+            m.cache = torch.zeros(rows, m.page_spec()["width"], dtype=dtype, device=self.device)
+            m.block_size = self.block_size
+        for m in states:
+            m.state = torch.zeros(slots, *m.state_spec()["shape"], dtype=torch.float32, device=self.device)
+        self.num_state_slots = slots
+
+    @torch.inference_mode()
+    def run_portions(self, plan, want=None, sample: bool = True):
+        """One step over (sequence, count) pairs as Scheduler.commit left them: the next ``count`` tokens of every
+        sequence, continuing from its pages and state slot; prompt pieces and single decoded tokens share the batch.
+
+        want is None: logits are computed where a sequence's known tokens end with this step, and (``sample``) a token
+        is drawn there -> one token id or None per pair.  want = per pair a list of positions inside its piece:
+        -> fp32 logits [wanted, vocab] in that order (None when nothing is wanted); nothing is sampled."""
+        bs = self.block_size
+        ids, pos, slots, seq_of, cu, past, state_slots = [], [], [], [], [0], [], []
+        for i, (seq, count) in enumerate(plan):
+            a, b = seq.num_computed_tokens, seq.num_computed_tokens + count
+            assert b <= seq.num_tokens and len(seq.block_table) * bs >= b
+            ids.extend(seq.token_ids[a:b])
+            pos.extend(range(a, b))
+            table = seq.block_table
+            slots.extend(table[p // bs] * bs + p % bs for p in range(a, b))
+            seq_of.extend([i] * count)
+            cu.append(cu[-1] + count)
+            past.append(a)
+            state_slots.append(seq.state_slot)
+        if want is None:
+            ends = [i for i, (seq, count) in enumerate(plan) if seq.num_computed_tokens + count == seq.num_tokens]
+            rows = [cu[i + 1] - 1 for i in ends]
+        else:
+            rows = [cu[i] + o for i, offsets in enumerate(want) for o in offsets]
+        to = lambda data, dt: self._to_device(torch.tensor(data, dtype=dt, device="cpu"))  # noqa: E731
+        set_context(True, cu_seqlens_q=to(cu, torch.int32), max_seqlen_q=max(c for _, c in plan),
+                    slot_mapping=to(slots, torch.int32), block_tables=self._prepare_block_tables([s for s, _ in plan]),
+                    past_lens=to(past, torch.int32), state_slots=to(state_slots, torch.int32),
+                    seq_of_token=to(seq_of, torch.int32))
+        try:
+            state = self.model(to(ids, torch.int64), to(pos, torch.int64))
+            if not rows:
+                torch.cuda.current_stream().synchronize()       # the pinned staging tensors die with this frame
+                return None if want is not None else [None] * len(plan)
+            rows_t = to(rows, torch.int32)
+            if want is not None or not sample:
+                logits = self.model.compute_logits(state, rows_t, out_dtype=torch.float32)
+                torch.cuda.current_stream().synchronize()
+                return logits
+            logits = self.model.compute_logits(state, rows_t, out_dtype=torch.bfloat16)
+            temperatures = to([plan[i][0].temperature for i in ends], torch.float32)
+            drawn = self.sampler(logits, temperatures).tolist()
+            tokens = [None] * len(plan)
+            for i, t in zip(ends, drawn):
+                tokens[i] = t
+            return tokens
+        finally:
+            reset_context()
+
     # ------------------------------------------------------------------ host -> device metadata
     def _to_device(self, t: torch.Tensor, device=None) -> torch.Tensor:
         device = device if device is not None else getattr(self, "device", None)
@@ -721,6 +802,7 @@ class ModelRunner:
             reset_context()
         self.graph_vars = g
 
+    portioned = False
     max_graph_bs = 0
     graph_has_head = False
     run_ahead = False

@@ -9,7 +9,7 @@ when the block pool is exhausted.
 
 from collections import deque
 
-from byox_vllm_amd.engine.block_manager import BlockManager
+from byox_vllm_amd.engine.block_manager import BlockManager, StateSlotManager
 from byox_vllm_amd.engine.sequence import Sequence, SequenceStatus
 from byox_vllm_amd.utils.logging import logger
 
@@ -22,6 +22,11 @@ class Scheduler:
         self.block_manager = BlockManager(config.num_kvcache_blocks, config.kvcache_block_size)
         self.waiting: deque[Sequence] = deque()
         self.running: deque[Sequence] = deque()
+        # portioned stepping (models that set it: Config.portioned): a step is a list of (sequence, token count) pairs,
+        # prompt pieces beside single decoded tokens; requests with a recurrent state also hold a state slot
+        self.portioned = bool(getattr(config, "portioned", False))
+        slots = getattr(config, "num_state_slots", 0)
+        self.state_slots = StateSlotManager(slots) if slots > 0 else None
         # Quiet decode steps.  After a full pass over the running queue the scheduler knows for how many further steps
         # that pass would repeat itself exactly: as long as the queues do not change, every scheduled sequence grows by
         # one token per step, and none of them reaches a block boundary (length % block_size in {0, 1}: a block to
@@ -102,7 +107,99 @@ class Scheduler:
         self._quiet_left = 0
         seq.status = SequenceStatus.WAITING
         self.block_manager.deallocate(seq)
+        if self.state_slots is not None:
+            self.state_slots.release(seq)
         self.waiting.appendleft(seq)
+
+    # -- portioned stepping -----------------------------------------------------
+    def commit(self, plan: list[tuple[Sequence, int]]) -> list[tuple[Sequence, int]]:
+        """Make a step of (sequence, count) pairs runnable: admit sequences that are still waiting (state slot), grow
+        their block tables to cover the tokens of this step.  The plan may come from schedule_portions (the engine's
+        own policy) or from a caller that replays a fixed schedule; both run through here and through
+        ModelRunner.run_portions.  Raises when the pools cannot hold the plan."""
+        for seq, count in plan:
+            assert 0 < count <= seq.num_tokens - seq.num_computed_tokens, f"{seq}: {count} tokens asked, " \
+                f"{seq.num_tokens - seq.num_computed_tokens} left"
+            if seq.status is SequenceStatus.WAITING:
+                if self.state_slots is not None:
+                    self.state_slots.allocate(seq)
+                seq.status = SequenceStatus.RUNNING
+                if seq in self.waiting:
+                    self.waiting.remove(seq)
+                self.running.append(seq)
+            self.block_manager.extend(seq, seq.num_computed_tokens + count)
+        return plan
+
+    def schedule_portions(self) -> list[tuple[Sequence, int]]:
+        """The engine's own policy for portioned stepping: every running request that is decoding gets its one token,
+        then prompts (running ones first, then waiting ones in arrival order) get as large a piece as the step's token
+        budget leaves.  Nothing is admitted that the block pool or the state slots cannot hold; when a decoding request
+        cannot get its next block, the youngest running request is preempted (its prompt is recomputed later)."""
+        budget = self.max_num_batched_tokens
+        bm = self.block_manager
+        plan: list[tuple[Sequence, int]] = []
+        free = len(bm.free_block_ids)
+        for seq in list(self.running):
+            if seq not in self.running:
+                continue                       # preempted below
+            left = seq.num_tokens - seq.num_computed_tokens
+            count = min(left, budget)
+            if count <= 0:
+                continue
+            need = bm.blocks_short(seq, seq.num_computed_tokens + count)
+            while need > free and self.running[-1] is not seq:
+                victim = self.running.pop()
+                plan = [(s, c) for s, c in plan if s is not victim]
+                self._preempt(victim)
+                free = len(bm.free_block_ids) - sum(bm.blocks_short(s, s.num_computed_tokens + c) for s, c in plan)
+            if need > free:
+                count = min(count, (len(seq.block_table) + free) * bm.block_size - seq.num_computed_tokens)
+                if count <= 0:
+                    continue
+                need = bm.blocks_short(seq, seq.num_computed_tokens + count)
+            plan.append((seq, count))
+            budget -= count
+            free -= need
+        admitted = 0
+        while self.waiting and budget > 0 and len(self.running) + admitted < self.max_num_seqs:
+            seq = self.waiting[0]
+            if self.state_slots is not None and len(self.state_slots.free) <= admitted:
+                break
+            count = min(seq.num_tokens - seq.num_computed_tokens, budget, free * bm.block_size)
+            if count <= 0:
+                break
+            self.waiting.popleft()             # commit() admits it: state slot, running queue, pages
+            plan.append((seq, count))
+            admitted += 1
+            budget -= count
+            free -= bm.blocks_short(seq, count)
+        return self.commit(plan)
+
+    def advance(self, plan: list[tuple[Sequence, int]], token_ids: list[int | None]) -> list[Sequence]:
+        """After a portioned step: count the tokens as computed; a request whose known tokens are all computed takes
+        the token sampled for it (None: a replayed request that is fed its tokens from outside).  -> finished."""
+        finished: list[Sequence] = []
+        for (seq, count), token_id in zip(plan, token_ids):
+            seq.num_computed_tokens += count
+            if seq.num_computed_tokens < seq.num_tokens or token_id is None:
+                continue
+            seq.append_token(token_id)
+            if (token_id == self.eos and not seq.ignore_eos) or seq.num_completion_tokens == seq.max_tokens:
+                self.finish(seq)
+                finished.append(seq)
+        return finished
+
+    def finish(self, seq: Sequence) -> None:
+        """The request is over: its pages and its state slot go back to the pools."""
+        seq.status = SequenceStatus.FINISHED
+        self.block_manager.deallocate(seq)
+        if self.state_slots is not None:
+            self.state_slots.release(seq)
+        if seq in self.running:
+            self.running.remove(seq)
+        if seq in self.waiting:
+            self.waiting.remove(seq)
+        self._quiet_left = 0
 
     def postprocess(self, seqs: list[Sequence], token_ids: list[int]) -> list[Sequence]:
         """Append the step's tokens; -> the sequences that finished with it (the reference returns nothing and has the

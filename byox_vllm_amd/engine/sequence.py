@@ -35,6 +35,10 @@ class Sequence:
         self.last_token = self.token_ids[-1]
         self.num_cached_tokens = 0
         self.block_table: list[int] = []
+        # portioned stepping (prompt pieces of any size, then single tokens): tokens whose cache rows / state updates
+        # are done, and the slot of the request's recurrent state (-1: none)
+        self.num_computed_tokens = 0
+        self.state_slot = -1
         self.temperature = sp.temperature
         self.max_tokens = sp.max_tokens
         self.ignore_eos = sp.ignore_eos
@@ -83,6 +87,12 @@ class Sequence:
         assert 0 <= i < self.num_blocks
         lo = i * self.block_size
         return self.token_ids[lo: lo + self.block_size]
+
+    def extend_tokens(self, token_ids: list[int]) -> None:
+        """More known tokens for a request whose text arrives in pieces (a replayed trace); they count as prompt."""
+        self.token_ids.extend(token_ids)
+        self.num_tokens = self.num_prompt_tokens = len(self.token_ids)
+        self.last_token = self.token_ids[-1]
 
     def append_token(self, token_id: int) -> None:
         self.token_ids.append(token_id)

@@ -431,3 +431,177 @@ def stage_decode_packed(packed, bs, bt_cols, g, prev_tokens=None, block_size=0):
                                        ptr(g["positions"]), ptr(g["slot_mapping"]), ptr(g["context_lens"]),
                                        ptr(g["block_tables"]), g["block_tables"].size(1), ptr(g.get("temperatures")),
                                        ptr(g.get("step")), stream()), "nv_stage_decode_packed")
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# Kernels of models with an fp32 residual stream (bf16 or true fp32 storage): nv_linear and its row-wise companions.
+
+EPI_NONE, EPI_GLU, EPI_SOFTCAP, EPI_ROW_GATE = 0, 1, 2, 3
+ACT_SILU, ACT_GELU_TANH = 0, 1
+
+
+def _code32(dt) -> int:
+    return dtype_code(dt, allow_f32=True)
+
+
+def linear(x, w, bias=None, out=None, out_dtype=None, *, rows=None, a_rows=None, batch=1, a_batch_stride=0,
+           w_batch_stride=0, out_batch_stride=0, group_offsets=None, max_group_rows=None, epilogue=EPI_NONE,
+           act=ACT_SILU, gate=None, gate_stride=0, cap=0.0, n=None):
+    """nv_linear.  ``x`` [M, >=K] (row stride free) in the model dtype, ``w`` [.., K] rows of the same dtype.
+    Plain: w [N, K] -> out [M, N].  ``batch`` > 1: per-batch element strides select the operands (heads).
+    ``group_offsets`` [batch + 1]: batch b owns output rows [off[b], off[b+1]) (experts), ``a_rows`` maps an output row to
+    its row of x, ``max_group_rows`` bounds a group.  GLU: w holds n gate rows then n up rows per batch."""
+    require_gpu(x, "linear")
+    assert x.dim() == 2 and x.stride(1) == 1 and w.stride(-1) == 1 and w.dtype == x.dtype and w.is_cuda
+    K = w.size(-1)
+    if n is None:
+        n = w.size(-2) // (2 if epilogue == EPI_GLU else 1)
+    M = x.size(0) if rows is None else rows
+    grid_rows = M if group_offsets is None else (max_group_rows if max_group_rows is not None else M)
+    out_dtype = out_dtype or x.dtype
+    if out is None:
+        cols = n * batch if (batch > 1 and group_offsets is None) else n
+        out = torch.empty(M, cols, dtype=out_dtype, device=x.device)
+        if batch > 1 and group_offsets is None and out_batch_stride == 0:
+            out_batch_stride = n
+    assert out.stride(-1) == 1 and out.dtype == out_dtype
+    if bias is not None:
+        assert bias.dtype == x.dtype and bias.is_contiguous()
+    if gate is not None:
+        assert gate.dtype == torch.float32
+    if group_offsets is not None:
+        assert group_offsets.dtype == torch.int32 and group_offsets.numel() == batch + 1
+    if a_rows is not None:
+        assert a_rows.dtype == torch.int32
+    check(lib().nv_linear(ptr(x), x.stride(0), ptr(a_rows), ptr(w), w.stride(-2), ptr(bias), ptr(out), out.stride(0),
+                          _code32(out_dtype), grid_rows, n, K, batch, a_batch_stride, w_batch_stride, out_batch_stride,
+                          n if bias is not None and batch > 1 else 0, ptr(group_offsets), epilogue, act, ptr(gate),
+                          gate_stride, cap, _code32(x.dtype), stream()), "nv_linear")
+    return out
+
+
+def embed_scale(ids, table, scale, out=None):
+    require_gpu(table, "embed_scale")
+    assert ids.dtype == torch.int64 and ids.is_contiguous() and table.is_contiguous()
+    T, width = ids.numel(), table.size(1)
+    out = torch.empty(T, width, dtype=torch.float32, device=table.device) if out is None else out
+    check(lib().nv_embed_scale(ptr(ids), ptr(table), ptr(out), T, width, table.size(0), scale, _code32(table.dtype),
+                               stream()), "nv_embed_scale")
+    return out
+
+
+def dyt_norm(x, alpha, w, b, delta=None, rows_idx=None, out=None):
+    """Dynamic Tanh of the fp32 residual rows ``x`` (updated in place by ``delta`` first when given)."""
+    require_gpu(x, "dyt_norm")
+    n = x.size(-1)
+    assert x.dtype == torch.float32 and x.is_contiguous() and alpha.dtype == torch.float32 and w.dtype == b.dtype
+    assert w.numel() == n and b.numel() == n
+    rows = x.size(0) if rows_idx is None else rows_idx.numel()
+    if delta is not None:
+        assert delta.dtype == torch.float32 and delta.stride(1) == 1 and delta.shape == x.shape
+    if rows_idx is not None:
+        assert rows_idx.dtype == torch.int32
+    out = torch.empty(rows, n, dtype=w.dtype, device=x.device) if out is None else out
+    check(lib().nv_dyt_norm(ptr(x), ptr(delta), delta.stride(0) if delta is not None else 0, ptr(rows_idx), ptr(alpha),
+                            ptr(w), ptr(b), ptr(out), rows, n, _code32(w.dtype), stream()), "nv_dyt_norm")
+    return out
+
+
+def rms_norm_f32(x, w, eps, out=None):
+    """RMS norm of fp32 rows (a column slice of a wider buffer is fine) -> rows in the dtype of ``w``."""
+    require_gpu(x, "rms_norm_f32")
+    assert x.dim() == 2 and x.dtype == torch.float32 and x.stride(1) == 1 and w.numel() == x.size(1)
+    out = torch.empty(x.shape, dtype=w.dtype, device=x.device) if out is None else out
+    check(lib().nv_rmsnorm_f32(ptr(x), x.stride(0), ptr(w), ptr(out), out.stride(0), x.size(0), x.size(1), eps,
+                               _code32(w.dtype), stream()), "nv_rmsnorm_f32")
+    return out
+
+
+def gla_recurrent(proj, offsets, z, state, cu_q, past_lens, state_slots, norm_w, heads, dim, vdim, tau, q_scale, eps,
+                  out=None):
+    """Gated linear attention over the step's tokens; ``proj`` fp32 [T, *] holds q | k | v | g at ``offsets``; ``state``
+    fp32 [slots, heads, dim, vdim] is read (unless the request starts) and written back."""
+    require_gpu(proj, "gla_recurrent")
+    T = proj.size(0)
+    assert proj.dtype == z.dtype == state.dtype == torch.float32 and proj.stride(1) == 1 and z.stride(1) == 1
+    assert state.is_contiguous() and state.shape[1:] == (heads, dim, vdim) and norm_w.numel() == vdim
+    assert cu_q.dtype == past_lens.dtype == state_slots.dtype == torch.int32
+    B = past_lens.numel()
+    assert cu_q.numel() == B + 1 and state_slots.numel() == B
+    out = torch.empty(T, heads * vdim, dtype=norm_w.dtype, device=proj.device) if out is None else out
+    q_off, k_off, v_off, g_off = offsets
+    check(lib().nv_gla_recurrent(ptr(proj), proj.stride(0), q_off, k_off, v_off, g_off, ptr(z), z.stride(0), ptr(state),
+                                 ptr(cu_q), ptr(past_lens), ptr(state_slots), ptr(norm_w), ptr(out), B, heads, dim, vdim,
+                                 tau, q_scale, eps, _code32(norm_w.dtype), stream()), "nv_gla_recurrent")
+    return out
+
+
+def latent_kv_store(kv, norm_w, positions, inv_freq, mscale, slot_mapping, cache, rank, rot_dim, rot_dims, eps):
+    require_gpu(kv, "latent_kv_store")
+    assert kv.dtype == torch.float32 and kv.stride(1) == 1 and kv.size(1) == rank + rot_dim
+    assert positions.dtype == torch.int64 and slot_mapping.dtype == torch.int32 and inv_freq.dtype == torch.float32
+    assert cache.is_contiguous() and cache.size(-1) == rank + rot_dim and cache.dtype == norm_w.dtype
+    assert positions.numel() == slot_mapping.numel() == kv.size(0) and inv_freq.numel() * 2 >= rot_dims
+    check(lib().nv_latent_kv_store(ptr(kv), kv.stride(0), ptr(norm_w), ptr(positions), ptr(inv_freq), mscale,
+                                   ptr(slot_mapping), ptr(cache), kv.size(0), rank, rot_dim, rot_dims, eps,
+                                   _code32(cache.dtype), stream()), "nv_latent_kv_store")
+
+
+def latent_q_rope(q, positions, inv_freq, mscale, qa, heads, dim, rot_dim, rot_dims, rank):
+    require_gpu(q, "latent_q_rope")
+    assert q.stride(1) == 1 and q.size(1) == heads * (dim + rot_dim) and qa.dtype == torch.float32 and qa.is_contiguous()
+    assert qa.numel() == q.size(0) * heads * (rank + rot_dim) and positions.dtype == torch.int64
+    check(lib().nv_latent_q_rope(ptr(q), q.stride(0), ptr(positions), ptr(inv_freq), mscale, ptr(qa), q.size(0), heads,
+                                 dim, rot_dim, rot_dims, rank, _code32(q.dtype), stream()), "nv_latent_q_rope")
+
+
+def latent_attn(qa, cache, block_tables, cu_q, past_lens, seq_of_token, heads, rank, rot_dim, block_size, window, scale,
+                out=None):
+    """Sliding-window attention of absorbed queries ``qa`` fp32 [T, heads, rank + rot_dim] over the paged latent cache
+    -> [T, heads * rank] in the cache dtype (sum of softmax weights times latents)."""
+    require_gpu(qa, "latent_attn")
+    T = qa.size(0)
+    assert qa.dtype == torch.float32 and qa.is_contiguous() and cache.is_contiguous()
+    assert block_tables.dtype == torch.int32 and block_tables.is_contiguous() and block_tables.dim() == 2
+    assert cu_q.dtype == past_lens.dtype == seq_of_token.dtype == torch.int32 and seq_of_token.numel() == T
+    out = torch.empty(T, heads * rank, dtype=cache.dtype, device=qa.device) if out is None else out
+    check(lib().nv_latent_attn(ptr(qa), ptr(cache), ptr(block_tables), block_tables.size(1), ptr(cu_q), ptr(past_lens),
+                               ptr(seq_of_token), ptr(out), T, heads, rank, rot_dim, block_size, window, scale,
+                               _code32(cache.dtype), stream()), "nv_latent_attn")
+    return out
+
+
+def moe_route(logits, experts, top):
+    """fp32 router logits [T, >=experts] -> (chosen experts int32 [T, top], softmax over the chosen logits fp32 [T, top])."""
+    require_gpu(logits, "moe_route")
+    assert logits.dtype == torch.float32 and logits.stride(1) == 1
+    T = logits.size(0)
+    idx = torch.empty(T, top, dtype=torch.int32, device=logits.device)
+    wt = torch.empty(T, top, dtype=torch.float32, device=logits.device)
+    check(lib().nv_moe_route(ptr(logits), logits.stride(0), ptr(idx), ptr(wt), T, experts, top, stream()), "nv_moe_route")
+    return idx, wt
+
+
+def moe_sort(idx, experts):
+    """-> (offsets int32 [experts + 1], token of every sorted row int32 [T * top], sorted row of every pair int32 [T, top])."""
+    T, top = idx.shape
+    dev = idx.device
+    offsets = torch.empty(experts + 1, dtype=torch.int32, device=dev)
+    sorted_token = torch.empty(T * top, dtype=torch.int32, device=dev)
+    slot_of = torch.empty(T, top, dtype=torch.int32, device=dev)
+    check(lib().nv_moe_sort(ptr(idx), T, experts, top, ptr(offsets), ptr(sorted_token), ptr(slot_of), stream()),
+          "nv_moe_sort")
+    return offsets, sorted_token, slot_of
+
+
+def moe_combine(y, slot_of, weights, shared=None, shared_gate=None, out=None):
+    T, top = slot_of.shape
+    width = y.size(1)
+    assert y.dtype == weights.dtype == torch.float32 and y.is_contiguous() and weights.is_contiguous()
+    if shared is not None:
+        assert shared.dtype == torch.float32 and shared.is_contiguous() and shared_gate.dtype == torch.float32
+    out = torch.empty(T, width, dtype=torch.float32, device=y.device) if out is None else out
+    check(lib().nv_moe_combine(ptr(y), ptr(slot_of), ptr(weights), top, ptr(shared), ptr(shared_gate),
+                               shared_gate.stride(0) if shared_gate is not None else 0, ptr(out), T, width, stream()),
+          "nv_moe_combine")
+    return out

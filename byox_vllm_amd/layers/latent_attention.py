@@ -1,0 +1,82 @@
+"""Latent attention mixer: keys and values of all heads are up-projections of one low-rank latent per token, so the
+cache holds per token only that latent c (kv_rank numbers, RMS-normed) and one rotated key part (rot_dim numbers)
+shared by the heads (the multi-head latent attention of DeepSeek-V2).  Scores of head h:
+
+    s = (q_nope[h] . (W_uk[h] c) + q_rot[h] . k_rot) * scale
+
+The up-projections never run over cached tokens: W_uk[h] is folded into the query (q_abs[h] = W_uk[h]^T q_nope[h], one
+small product per head and step token) and W_uv[h] is applied to the attention-weighted sum of latents.  Attention is
+then multi-query attention over rows [c | k_rot] with a sliding window: position i sees j with 0 <= i - j < window.
+Queries go through a latent of their own (RMS-normed), each head's output is multiplied by sigmoid(W_g h)[head].
+
+A layer built with ``kv_source`` has no key/value down-projection: it reads the cache rows another layer wrote in the
+same step (same kv_rank, rot_dim and rotation), with its own W_uk, W_uv, queries and window.
+
+Cache rows live in pages of the engine's BlockManager ([pages * block_size, kv_rank + rot_dim] in the model dtype);
+scores, softmax and the weighted sum are fp32 (csrc/latent_attn.hip)."""
+
+import torch
+from torch import nn
+
+from byox_vllm_amd import kernels
+from byox_vllm_amd.layers.linear import DenseLinear
+from byox_vllm_amd.layers.rotary_embedding import scaled_inv_freq
+from byox_vllm_amd.utils.context import get_context
+
+
+class LatentAttention(nn.Module):
+    def __init__(self, width: int, heads: int, dim: int, rot_dim: int, vdim: int, q_rank: int, kv_rank: int, scale: float,
+                 window: int, rot_dims: int, rot_base: float, rot_scaling: dict | None, eps: float,
+                 kv_source: "LatentAttention | None" = None):
+        super().__init__()
+        self.heads, self.dim, self.rot_dim, self.vdim = heads, dim, rot_dim, vdim
+        self.q_rank, self.kv_rank, self.scale, self.window, self.rot_dims, self.eps = q_rank, kv_rank, scale, window, rot_dims, eps
+        assert rot_dims <= rot_dim and rot_dims % 2 == 0
+        self.own_kv = kv_source is None
+        object.__setattr__(self, "kv_source", kv_source)      # a reference, not a submodule
+        if kv_source is not None:
+            assert (kv_source.kv_rank, kv_source.rot_dim, kv_source.own_kv) == (kv_rank, rot_dim, True)
+        shards = {"dq": q_rank}
+        if self.own_kv:
+            shards["dkv"] = kv_rank + rot_dim
+        shards["g"] = heads
+        self.down = DenseLinear(width, shards=shards)
+        self.dq_norm = nn.Parameter(torch.ones(q_rank), requires_grad=False)
+        self.uq = DenseLinear(q_rank, heads * (dim + rot_dim))
+        if self.own_kv:
+            self.dkv_norm = nn.Parameter(torch.ones(kv_rank), requires_grad=False)
+        # W_uk per head, stored transposed ([heads, kv_rank, dim]) so that folding it into the query is a plain product
+        self.uk_t = nn.Parameter(torch.empty(heads, kv_rank, dim), requires_grad=False)
+        self.uk_t.weight_loader = lambda p, t: p.data.copy_(t.view(heads, dim, kv_rank).transpose(1, 2))
+        self.uv = DenseLinear(kv_rank, heads * vdim)
+        self.o = DenseLinear(heads * vdim, width)
+        inv_freq, self.magnitude = scaled_inv_freq(rot_dims, rot_base, rot_scaling)
+        self.register_buffer("inv_freq", inv_freq.to(torch.float32), persistent=False)
+        self.cache = torch.tensor([])          # [pages * block_size, kv_rank + rot_dim], bound by the runner
+        self.block_size = 0
+
+    def page_spec(self) -> dict | None:
+        return {"width": self.kv_rank + self.rot_dim} if self.own_kv else None
+
+    def forward(self, h: torch.Tensor, positions: torch.Tensor) -> torch.Tensor:
+        ctx = get_context()
+        H, d, r, R = self.heads, self.dim, self.rot_dim, self.kv_rank
+        inv_freq = self.inv_freq if self.inv_freq.dtype == torch.float32 else self.inv_freq.float()
+        dn = self.down(h, out_dtype=torch.float32)
+        q = self.uq(kernels.rms_norm_f32(dn[:, :self.q_rank], self.dq_norm.data, self.eps))
+        if self.own_kv:
+            at = self.down.offset("dkv")
+            kernels.latent_kv_store(dn[:, at: at + R + r], self.dkv_norm.data, positions, inv_freq, self.magnitude,
+                                    ctx.slot_mapping, self.cache, R, r, self.rot_dims, self.eps)
+        src = self if self.own_kv else self.kv_source
+        T = h.size(0)
+        qa = torch.empty(T, H * (R + r), dtype=torch.float32, device=h.device)
+        kernels.linear(q, self.uk_t.data, out=qa, out_dtype=torch.float32, batch=H, a_batch_stride=d + r,
+                       w_batch_stride=R * d, out_batch_stride=R + r, n=R)
+        kernels.latent_q_rope(q, positions, inv_freq, self.magnitude, qa, H, d, r, self.rot_dims, R)
+        mix = kernels.latent_attn(qa, src.cache, ctx.block_tables, ctx.cu_seqlens_q, ctx.past_lens, ctx.seq_of_token,
+                                  H, R, r, src.block_size, self.window, self.scale)
+        o = kernels.linear(mix, self.uv.weight.data, batch=H, a_batch_stride=R, w_batch_stride=self.vdim * R,
+                           out_batch_stride=self.vdim, n=self.vdim, epilogue=kernels.EPI_ROW_GATE,
+                           gate=dn[:, self.down.offset("g"):], gate_stride=dn.stride(0))
+        return self.o(o, out_dtype=torch.float32)

@@ -367,3 +367,41 @@ class RowParallelLinear(LinearBase):
         if collectives_on(self.tp_size):
             tp_all_reduce(y)
         return y
+
+
+class DenseLinear(nn.Module):
+    """Unsharded linear layer on nv_linear: any in/out size, bf16 or fp32 parameters, fp32 accumulation; the output
+    dtype is chosen per call (fp32 where the consumer computes in fp32).  ``shards`` names row blocks that a checkpoint
+    stores as separate matrices (merged projections read the same input once): weight_loader(param, tensor, name)
+    copies one of them into place."""
+
+    def __init__(self, input_size: int, output_size: int | None = None, bias: bool = False,
+                 shards: dict[str, int] | None = None):
+        super().__init__()
+        self.row_of, at = {}, 0
+        for name, rows in (shards or {}).items():
+            self.row_of[name] = (at, rows)
+            at += rows
+        output_size = at if shards else output_size
+        self.weight = nn.Parameter(torch.empty(output_size, input_size), requires_grad=False)
+        self.weight.weight_loader = self.weight_loader
+        if bias:
+            self.bias = nn.Parameter(torch.empty(output_size), requires_grad=False)
+            self.bias.weight_loader = self.weight_loader
+        else:
+            self.register_parameter("bias", None)
+
+    def offset(self, shard: str) -> int:
+        return self.row_of[shard][0]
+
+    def weight_loader(self, param: nn.Parameter, loaded_weight: torch.Tensor, shard: str | None = None):
+        if shard is None:
+            assert param.shape == loaded_weight.shape, f"{tuple(param.shape)} != {tuple(loaded_weight.shape)}"
+            param.data.copy_(loaded_weight)
+        else:
+            at, rows = self.row_of[shard]
+            assert loaded_weight.shape[0] == rows and loaded_weight.shape[1:] == param.shape[1:]
+            param.data[at: at + rows].copy_(loaded_weight)
+
+    def forward(self, x, out_dtype=None, **kw):
+        return kernels.linear(x, self.weight.data, None if self.bias is None else self.bias.data, out_dtype=out_dtype, **kw)

@@ -19,6 +19,11 @@ class Context:
     slot_mapping: torch.Tensor | None = None
     context_lens: torch.Tensor | None = None
     block_tables: torch.Tensor | None = None
+    # portioned steps (prompt pieces and decoded tokens in one batch): per request the tokens it already holds and its
+    # state slot, per token the request it belongs to
+    past_lens: torch.Tensor | None = None
+    state_slots: torch.Tensor | None = None
+    seq_of_token: torch.Tensor | None = None
 
 
 _CONTEXT = Context()
@@ -29,10 +34,11 @@ def get_context() -> Context:
 
 
 def set_context(is_prefill, cu_seqlens_q=None, cu_seqlens_k=None, max_seqlen_q=0, max_seqlen_k=0,
-                slot_mapping=None, context_lens=None, block_tables=None) -> None:
+                slot_mapping=None, context_lens=None, block_tables=None, past_lens=None, state_slots=None,
+                seq_of_token=None) -> None:
     global _CONTEXT
     _CONTEXT = Context(is_prefill, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,
-                       slot_mapping, context_lens, block_tables)
+                       slot_mapping, context_lens, block_tables, past_lens, state_slots, seq_of_token)
 
 
 def reset_context() -> None:

@@ -36,6 +36,17 @@ def _load_quantized(model, packed, pending, name, tensor, quantization):
 
 
 def _load_one(model, packed, name, tensor):
+    target = getattr(model, "checkpoint_target", None)
+    if target is not None:       # the model names its own checkpoint tensors: (parameter path, shard id)
+        found = target(name)
+        assert found is not None, f"{name}: not a tensor of this model"
+        param = model.get_parameter(found[0])
+        loader = getattr(param, "weight_loader", default_weight_loader)
+        if found[1] is None:
+            loader(param, tensor)
+        else:
+            loader(param, tensor, found[1])
+        return
     for hf_key, (packed_key, shard_id) in packed.items():
         if hf_key in name:
             param = model.get_parameter(name.replace(hf_key, packed_key))
@@ -89,7 +100,11 @@ def init_random_weights(model: nn.Module, seed: int = 0) -> None:
     tests load an explicit state dict instead."""
     gens: dict = {}
     for name, param in model.named_parameters():
-        if name == "lm_head.weight" and param.data_ptr() == model.model.embed_tokens.weight.data_ptr():
+        if name == "lm_head.weight" and hasattr(model, "model") and \
+                param.data_ptr() == model.model.embed_tokens.weight.data_ptr():
+            continue
+        if name.endswith((".b", ".bias")) and "norm" in name:
+            param.data.zero_()
             continue
         if "norm" in name:
             param.data.fill_(1.0)

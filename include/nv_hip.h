@@ -35,6 +35,7 @@ extern "C" {
 
 #define NV_BF16 0
 #define NV_F16 1
+#define NV_F32 2 /* true 32-bit storage: taken by the entry points that say so (nv_linear and the fp32-residual kernels) */
 
 /* weight formats of nv_gemm */
 #define NV_W_DENSE 0 /* [N, K] row-major in the model dtype (reference layout, linear.py:24) */
@@ -324,6 +325,62 @@ int nv_allreduce(nv_comm_t* comm, const void* x, const float* partials, int num_
 int nv_allreduce_add_rmsnorm(nv_comm_t* comm, const void* x, const float* partials, int num_partials,
                              const void* residual, const void* weight, void* out, void* residual_out, int64_t rows,
                              int hidden, float eps, int dtype, nv_stream_t stream);
+
+/* ---- kernels of models that keep the residual stream in fp32 and run in bf16 or true fp32 (dtype NV_BF16 / NV_F32) ----
+ *
+ * nv_linear: out[b][m][n] = epilogue(sum_k A[b][row(m)][k] * W[b][n][k] + bias[b][n]), fp32 accumulation.  Any M, N, K.
+ *   a_rows       optional gather: row(m) = a_rows[m] (else m);
+ *   batch        independent products (one weight per head) with element strides per batch;
+ *   group_offsets  when given, batch b covers the output rows [group_offsets[b], group_offsets[b+1]) (one weight per
+ *                expert over rows sorted by expert); M then bounds the rows of one group;
+ *   epilogue     0 none; 1 gated unit: W holds N gate rows followed by N up rows, out = act(gate) * up with act = SiLU
+ *                (act 0) or the tanh form of GELU (act 1); 2 soft cap: c * tanh(out / c), c = epi_const;
+ *                3 row gate: out *= sigmoid(epi_ptr[m * epi_row_stride + b]);
+ *   out_dtype    NV_BF16 or NV_F32, independent of the operands' dtype. */
+int nv_linear(const void* a, int64_t a_row_stride, const int32_t* a_rows, const void* w, int64_t w_row_stride,
+              const void* bias, void* out, int64_t out_row_stride, int out_dtype, int64_t M, int N, int K, int batch,
+              int64_t a_batch_stride, int64_t w_batch_stride, int64_t out_batch_stride, int64_t bias_batch_stride,
+              const int32_t* group_offsets, int epilogue, int act, const float* epi_ptr, int64_t epi_row_stride,
+              float epi_const, int dtype, nv_stream_t stream);
+
+/* out[t] = table[ids[t]] * scale as fp32 rows (the residual stream's first value). */
+int nv_embed_scale(const int64_t* ids, const void* table, float* out, int64_t tokens, int width, int64_t vocab,
+                   float scale, int dtype, nv_stream_t stream);
+
+/* Dynamic Tanh: out = tanh(alpha * x) * w + b, element-wise, no statistics.  With `delta` the fp32 residual rows x are
+ * first updated in place (x += delta); with `rows_idx` output row i is computed from x row rows_idx[i]. */
+int nv_dyt_norm(float* x, const float* delta, int64_t delta_row_stride, const int32_t* rows_idx, const float* alpha,
+                const void* w, const void* b, void* out, int64_t rows, int n, int dtype, nv_stream_t stream);
+
+/* RMS norm of fp32 rows: out = x / sqrt(mean(x^2) + eps) * w, rounded to the storage type. */
+int nv_rmsnorm_f32(const float* x, int64_t x_row_stride, const void* w, void* out, int64_t out_row_stride, int64_t rows,
+                   int n, float eps, int dtype, nv_stream_t stream);
+
+/* Gated linear attention over this step's tokens of each request, state carried in fp32 slots (csrc/gla.hip). */
+int nv_gla_recurrent(const float* proj, int64_t proj_row_stride, int q_off, int k_off, int v_off, int g_off,
+                     const float* z, int64_t z_row_stride, float* state, const int32_t* cu_q, const int32_t* past_lens,
+                     const int32_t* state_slots, const void* norm_w, void* out, int num_seqs, int heads, int dim,
+                     int vdim, float tau, float q_scale, float eps, int dtype, nv_stream_t stream);
+
+/* Latent attention (csrc/latent_attn.hip): cache rows [kv_rank | rot_dim] per token, shared by all heads. */
+int nv_latent_kv_store(const float* kv, int64_t kv_row_stride, const void* norm_w, const int64_t* positions,
+                       const float* inv_freq, float mscale, const int32_t* slot_mapping, void* cache, int64_t tokens,
+                       int rank, int rot_dim, int rot_dims, float eps, int dtype, nv_stream_t stream);
+int nv_latent_q_rope(const void* q, int64_t q_row_stride, const int64_t* positions, const float* inv_freq, float mscale,
+                     float* qa, int64_t tokens, int heads, int dim, int rot_dim, int rot_dims, int rank, int dtype,
+                     nv_stream_t stream);
+int nv_latent_attn(const float* qa, const void* cache, const int32_t* block_tables, int table_cols, const int32_t* cu_q,
+                   const int32_t* past_lens, const int32_t* seq_of_token, void* out, int64_t tokens, int heads, int rank,
+                   int rot_dim, int block_size, int window, float scale, int dtype, nv_stream_t stream);
+
+/* Mixture of experts (csrc/moe.hip): routing, ordering by expert, weighted combination. */
+int nv_moe_route(const float* logits, int64_t row_stride, int32_t* idx, float* weights, int64_t tokens, int experts,
+                 int top, nv_stream_t stream);
+int nv_moe_sort(const int32_t* idx, int64_t tokens, int experts, int top, int32_t* offsets, int32_t* sorted_token,
+                int32_t* slot_of, nv_stream_t stream);
+int nv_moe_combine(const float* y, const int32_t* slot_of, const float* weights, int top, const float* shared,
+                   const float* shared_gate, int64_t shared_gate_stride, float* out, int64_t tokens, int width,
+                   nv_stream_t stream);
 
 #ifdef __cplusplus
 }
