@@ -16,7 +16,8 @@ __global__ __launch_bounds__(256) void embed_scale_kernel(const int64_t* __restr
   for (int i = threadIdx.x; i < width; i += blockDim.x) out[t * width + i] = ld_f32<T>(row + i) * scale;
 }
 
-// x[r] += delta[r] (when delta is given; written back), out[i] = tanh(alpha * x[r]) * w + b with r = rows_idx ? rows_idx[i] : i
+// v = x[r] + delta[r] (when delta is given; written back to x unless rows are gathered), out[i] = tanh(alpha * v) * w + b
+// with r = rows_idx ? rows_idx[i] : i
 template <typename T>
 __global__ __launch_bounds__(256) void dyt_kernel(float* __restrict__ x, const float* __restrict__ delta,
                                                   int64_t delta_rs, const int32_t* __restrict__ rows_idx,
@@ -30,7 +31,7 @@ __global__ __launch_bounds__(256) void dyt_kernel(float* __restrict__ x, const f
     float v = xr[j];
     if (delta) {
       v += delta[r * delta_rs + j];
-      xr[j] = v;
+      if (!rows_idx) xr[j] = v;
     }
     st_f32<T>(out + i * n + j, tanhf(a * v) * ld_f32<T>(w + j) + ld_f32<T>(b + j));
   }
@@ -69,7 +70,6 @@ extern "C" int nv_dyt_norm(float* x, const float* delta, int64_t delta_row_strid
                            nv_stream_t stream) {
   NV_CHECK_ARG(x && alpha && w && b && out, "nv_dyt_norm: null pointer");
   NV_CHECK_ARG(dtype == NV_BF16 || dtype == NV_F32, "nv_dyt_norm: bad dtype %d", dtype);
-  NV_CHECK_ARG(!(delta && rows_idx), "nv_dyt_norm: the residual add and the row gather exclude each other");
   NV_CHECK_ARG(rows >= 0 && n > 0, "nv_dyt_norm: bad shape");
   if (rows == 0) return NV_OK;
   NV_DISPATCH_T(dtype, dyt_kernel<T><<<dim3((unsigned)rows), dim3(256), 0, (hipStream_t)stream>>>(

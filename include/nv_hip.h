@@ -348,7 +348,8 @@ int nv_embed_scale(const int64_t* ids, const void* table, float* out, int64_t to
                    float scale, int dtype, nv_stream_t stream);
 
 /* Dynamic Tanh: out = tanh(alpha * x) * w + b, element-wise, no statistics.  With `delta` the fp32 residual rows x are
- * first updated in place (x += delta); with `rows_idx` output row i is computed from x row rows_idx[i]. */
+ * first updated in place (x += delta); with `rows_idx` output row i is computed from x row rows_idx[i] (plus that row of
+ * delta), and x is left as it is. */
 int nv_dyt_norm(float* x, const float* delta, int64_t delta_row_stride, const int32_t* rows_idx, const float* alpha,
                 const void* w, const void* b, void* out, int64_t rows, int n, int dtype, nv_stream_t stream);
 
