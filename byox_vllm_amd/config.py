@@ -90,7 +90,8 @@ class Config:
         if self.portioned and self.num_state_slots <= 0:
             self.num_state_slots = self.max_num_seqs
         self.max_model_len = min(self.max_model_len, self.hf_config.max_position_embeddings)
-        assert self.max_num_batched_tokens >= self.max_model_len
+        # a step must hold a whole prompt, except where prompts are stepped through in portions
+        assert self.portioned or self.max_num_batched_tokens >= self.max_model_len
 
 
 def qwen2_config(name: str, dtype=torch.bfloat16, **overrides):

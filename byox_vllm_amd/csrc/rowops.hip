@@ -51,7 +51,68 @@ __global__ __launch_bounds__(256) void rmsnorm_f32_kernel(const float* __restric
   for (int j = threadIdx.x; j < n; j += blockDim.x) st_f32<T>(out + r * out_rs + j, xr[j] * inv * ld_f32<T>(w + j));
 }
 
+// Gumbel-max sampling from fp32 logits: argmax_j (l_j / T + g_j) with g_j = -log(-log(u_j)), u_j a hash of (seed, row,
+// column); temperature 0 takes the plain argmax.  Ties go to the lowest index.
+__device__ __forceinline__ uint32_t mix32(uint64_t x) {
+  x ^= x >> 33;
+  x *= 0xff51afd7ed558ccdULL;
+  x ^= x >> 33;
+  x *= 0xc4ceb9fe1a85ec53ULL;
+  x ^= x >> 33;
+  return (uint32_t)x;
+}
+
+__global__ __launch_bounds__(256) void sample_f32_kernel(const float* __restrict__ logits, int64_t rs,
+                                                         const float* __restrict__ temperatures,
+                                                         int64_t* __restrict__ tokens, int V, uint64_t seed) {
+  __shared__ float bv[256];
+  __shared__ int bi[256];
+  const int row = blockIdx.x;
+  const float temp = temperatures[row];
+  const float* l = logits + row * rs;
+  float best = -INFINITY;
+  int arg = V;
+  for (int j = threadIdx.x; j < V; j += blockDim.x) {
+    float v = l[j];
+    if (temp > 0.0f) {
+      const uint32_t h = mix32(seed * 0x9E3779B97F4A7C15ULL + ((uint64_t)row << 32) + (uint64_t)j);
+      const float u = ((float)(h >> 8) + 0.5f) * (1.0f / 16777216.0f);
+      v = v / temp - logf(-logf(u));
+    }
+    if (v > best || arg == V) {
+      best = v;
+      arg = j;
+    }
+  }
+  bv[threadIdx.x] = best;
+  bi[threadIdx.x] = arg;
+  __syncthreads();
+  for (int o = 128; o > 0; o >>= 1) {
+    if ((int)threadIdx.x < o) {
+      const float v2 = bv[threadIdx.x + o];
+      const int i2 = bi[threadIdx.x + o];
+      if (i2 < V && (bi[threadIdx.x] >= V || v2 > bv[threadIdx.x] || (v2 == bv[threadIdx.x] && i2 < bi[threadIdx.x]))) {
+        bv[threadIdx.x] = v2;
+        bi[threadIdx.x] = i2;
+      }
+    }
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) tokens[row] = bi[0];
+}
+
 }  // namespace
+
+extern "C" int nv_sample_f32(const float* logits, int64_t row_stride, const float* temperatures, int64_t* tokens, int B,
+                             int V, uint64_t seed, nv_stream_t stream) {
+  NV_CHECK_ARG(logits && temperatures && tokens, "nv_sample_f32: null pointer");
+  NV_CHECK_ARG(B >= 0 && V > 0, "nv_sample_f32: bad shape B=%d V=%d", B, V);
+  if (B == 0) return NV_OK;
+  sample_f32_kernel<<<dim3((unsigned)B), dim3(256), 0, (hipStream_t)stream>>>(logits, row_stride, temperatures, tokens, V,
+                                                                              seed);
+  NV_CHECK_LAUNCH();
+  return NV_OK;
+}
 
 extern "C" int nv_embed_scale(const int64_t* ids, const void* table, float* out, int64_t tokens, int width, int64_t vocab,
                               float scale, int dtype, nv_stream_t stream) {

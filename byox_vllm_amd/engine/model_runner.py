@@ -578,11 +578,10 @@ class ModelRunner:
                 torch.cuda.current_stream().synchronize()       # the pinned staging tensors die with this frame
                 return None if want is not None else [None] * len(plan)
             rows_t = to(rows, torch.int32)
+            logits = self.model.compute_logits(state, rows_t, out_dtype=torch.float32)
             if want is not None or not sample:
-                logits = self.model.compute_logits(state, rows_t, out_dtype=torch.float32)
                 torch.cuda.current_stream().synchronize()
                 return logits
-            logits = self.model.compute_logits(state, rows_t, out_dtype=torch.bfloat16)
             temperatures = to([plan[i][0].temperature for i in ends], torch.float32)
             drawn = self.sampler(logits, temperatures).tolist()
             tokens = [None] * len(plan)

@@ -517,6 +517,18 @@ def rms_norm_f32(x, w, eps, out=None):
     return out
 
 
+def sample_f32(logits, temperatures, seed=0, out=None):
+    """Tokens from fp32 logits [B, V]: argmax where the temperature is 0, Gumbel-max otherwise."""
+    require_gpu(logits, "sample_f32")
+    B, V = logits.shape
+    assert logits.dtype == torch.float32 and logits.stride(1) == 1
+    assert temperatures.dtype == torch.float32 and temperatures.numel() == B
+    out = torch.empty(B, dtype=torch.int64, device=logits.device) if out is None else out
+    check(lib().nv_sample_f32(ptr(logits), logits.stride(0), ptr(temperatures), ptr(out), B, V,
+                              seed & 0xFFFFFFFFFFFFFFFF, stream()), "nv_sample_f32")
+    return out
+
+
 def gla_recurrent(proj, offsets, z, state, cu_q, past_lens, state_slots, norm_w, heads, dim, vdim, tau, q_scale, eps,
                   out=None):
     """Gated linear attention over the step's tokens; ``proj`` fp32 [T, *] holds q | k | v | g at ``offsets``; ``state``

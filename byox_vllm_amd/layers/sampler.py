@@ -19,4 +19,7 @@ class Sampler(nn.Module):
 
     def forward(self, logits: torch.Tensor, temperatures: torch.Tensor, noise: torch.Tensor | None = None):
         self.calls += 1
+        if logits.dtype == torch.float32:      # models that hand over fp32 logits (fp32 residual stream)
+            assert noise is None
+            return kernels.sample_f32(logits, temperatures, seed=(self.seed << 32) + self.calls)
         return kernels.sample(logits, temperatures, noise=noise, seed=(self.seed << 32) + self.calls)

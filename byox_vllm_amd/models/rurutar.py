@@ -176,6 +176,8 @@ class RurutarForCausalLM(nn.Module):
         layer = self.layers[i]
         for norm in ("norm1", "norm2"):
             if rest == norm or rest.startswith(norm + "."):
+                if getattr(layer, norm) is None:
+                    return None, None          # a layer without a feed-forward has no second norm to feed
                 return base + norm + "." + self._norm_part(rest[len(norm):]), None
         part, _, leaf = rest.partition(".")
         if part == "mix":

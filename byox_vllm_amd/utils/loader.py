@@ -40,6 +40,8 @@ def _load_one(model, packed, name, tensor):
     if target is not None:       # the model names its own checkpoint tensors: (parameter path, shard id)
         found = target(name)
         assert found is not None, f"{name}: not a tensor of this model"
+        if found[0] is None:         # a tensor the configuration leaves without a consumer
+            return
         param = model.get_parameter(found[0])
         loader = getattr(param, "weight_loader", default_weight_loader)
         if found[1] is None:
@@ -72,7 +74,12 @@ def load_model(model: nn.Module, path: str, quantization: str | None = None):
 
 
 def load_state_dict_packed(model: nn.Module, weights: dict, cfg) -> None:
-    """Load a dict keyed by the packed names (qkv_proj / gate_up_proj hold the FULL, unsharded tensors)."""
+    """Load a dict keyed by the packed names (qkv_proj / gate_up_proj hold the FULL, unsharded tensors).  For a model
+    that names its own checkpoint tensors (``checkpoint_target``) the dict is keyed by those names."""
+    if getattr(model, "checkpoint_target", None) is not None:
+        for name, w in weights.items():
+            _load_one(model, {}, name, w)
+        return
     d = cfg.head_dim
     nq, nkv = cfg.num_attention_heads * d, cfg.num_key_value_heads * d
     tied = getattr(cfg, "tie_word_embeddings", False)

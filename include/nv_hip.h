@@ -357,6 +357,11 @@ int nv_dyt_norm(float* x, const float* delta, int64_t delta_row_stride, const in
 int nv_rmsnorm_f32(const float* x, int64_t x_row_stride, const void* w, void* out, int64_t out_row_stride, int64_t rows,
                    int n, float eps, int dtype, nv_stream_t stream);
 
+/* Sampler over fp32 logits: temperature 0 -> argmax (lowest index on ties), else Gumbel-max with noise hashed from
+ * (seed, row, column). */
+int nv_sample_f32(const float* logits, int64_t row_stride, const float* temperatures, int64_t* tokens, int B, int V,
+                  uint64_t seed, nv_stream_t stream);
+
 /* Gated linear attention over this step's tokens of each request, state carried in fp32 slots (csrc/gla.hip). */
 int nv_gla_recurrent(const float* proj, int64_t proj_row_stride, int q_off, int k_off, int v_off, int g_off,
                      const float* z, int64_t z_row_stride, float* state, const int32_t* cu_q, const int32_t* past_lens,
