@@ -139,6 +139,7 @@ class Scheduler:
         bm = self.block_manager
         plan: list[tuple[Sequence, int]] = []
         free = len(bm.free_block_ids)
+        preempted = False
         for seq in list(self.running):
             if seq not in self.running:
                 continue                       # preempted below
@@ -151,6 +152,7 @@ class Scheduler:
                 victim = self.running.pop()
                 plan = [(s, c) for s, c in plan if s is not victim]
                 self._preempt(victim)
+                preempted = True
                 free = len(bm.free_block_ids) - sum(bm.blocks_short(s, s.num_computed_tokens + c) for s, c in plan)
             if need > free:
                 count = min(count, (len(seq.block_table) + free) * bm.block_size - seq.num_computed_tokens)
@@ -161,7 +163,8 @@ class Scheduler:
             budget -= count
             free -= need
         admitted = 0
-        while self.waiting and budget > 0 and len(self.running) + admitted < self.max_num_seqs:
+        # a step that had to take pages away admits nobody: the preempted request would come straight back
+        while not preempted and self.waiting and budget > 0 and len(self.running) + admitted < self.max_num_seqs:
             seq = self.waiting[0]
             if self.state_slots is not None and len(self.state_slots.free) <= admitted:
                 break
