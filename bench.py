@@ -282,6 +282,86 @@ def run_generate_workload(args):
     print(json.dumps(line), flush=True)
 
 
+# --arch-compare: the Rurutar design beside the closest model family the engine has (the dense Qwen3 decoder) at equal
+# width, depth, active feed-forward size and vocabulary, both through LLM.generate: prefill and decode tokens/s.
+# name: (width, layers, prompts, prompt length, decoded tokens)
+ARCH_COMPARE_SIZES = {
+    "w1024": (1024, 8, 8, 2048, 64),
+    "w2048": (2048, 8, 8, 2048, 64),
+}
+
+
+def rurutar_bench_config(width: int, layers: int, vocab: int = 32000):
+    """A Rurutar configuration with the proportions of a real model's layers: two of three layers recurrent, every
+    third one latent attention over a sliding window (the second borrows the first one's cache rows), a dense first
+    feed-forward and mixtures after it whose active size equals the dense comparator's."""
+    from byox_vllm_amd.models.rurutar import rurutar_config
+    heads = width // 128
+    ff = 3 * width
+    experts, top, expert_ff, shared_ff = 16, 2, width, width                 # 2 * width + width active
+    gla = {"type": "gla", "mixer": {"heads": heads, "dim": 64, "vdim": 128, "tau": 16.0, "decay_rank": 32}}
+    lat = {"type": "latent_attention",
+           "mixer": {"heads": heads, "dim": 96, "rot_dim": 32, "vdim": 128, "kv_rank": width // 4, "q_rank": width // 2,
+                     "mask": {"size": 512}, "scale": 128 ** -0.5,
+                     "rot": {"base": 10000.0, "dims": 32,
+                             "scaling": {"factor": 8.0, "original": 1024, "fast": 32.0, "slow": 1.0}}}}
+    moe = {"kind": "moe", "router": {"experts": experts, "top": top}, "expert": {"ff": expert_ff}, "shared": {"ff": shared_ff}}
+    specs, first_latent = [], None
+    for i in range(layers):
+        layer = json.loads(json.dumps(lat if i % 3 == 1 else gla))
+        if i % 3 == 1:
+            if first_latent is None:
+                first_latent = i
+            elif (i // 3) % 2 == 1:
+                layer["mixer"]["kv_from"] = first_latent
+        layer["mlp"] = {"kind": "dense", "ff": ff} if i == 0 else moe
+        specs.append(layer)
+    raw = {"architecture": "Rurutar", "vocab": vocab, "width": width, "embedding": {"scale": 1.0}, "norm": {"eps": 1e-5},
+           "logit_softcap": 30.0, "layers": specs}
+    return rurutar_config(raw, None, dtype=torch.bfloat16)
+
+
+def run_arch_compare(args):
+    from byox_vllm_amd import LLM, SamplingParams
+    from byox_vllm_amd.config import qwen2_config
+    assert args.gpus == 1, "--arch-compare runs on one GPU"
+    random.seed(0)
+    results = []
+    for name, (width, layers, num, plen, decoded) in ARCH_COMPARE_SIZES.items():
+        if args.arch_sizes and name not in args.arch_sizes.split(","):
+            continue
+        params = SamplingParams(temperature=0.0, ignore_eos=True, max_tokens=decoded)
+        blocks = num * ((plen + decoded) // 256 + 2)
+        dense = qwen2_config("qwen3-0.6b", dtype=torch.bfloat16, hidden_size=width, intermediate_size=3 * width,
+                             num_hidden_layers=layers, num_attention_heads=width // 128, num_key_value_heads=width // 256,
+                             head_dim=128, vocab_size=32000, tie_word_embeddings=False)
+        row = {"size": name, "width": width, "layers": layers, "prompts": num, "prompt_len": plen, "decoded": decoded}
+        for label, hf in (("rurutar", rurutar_bench_config(width, layers)), ("qwen3_dense", dense)):
+            llm = LLM("synthetic", hf_config=hf, enforce_eager=args.eager, max_model_len=plen + decoded + 8,
+                      max_num_seqs=num, max_num_batched_tokens=num * plen, kvcache_block_size=256,
+                      num_kvcache_blocks=blocks)
+            runs = []
+            for i in range(1 + max(1, min(args.steps, 3))):
+                # fresh prompts every run: the dense model's prefix cache would otherwise serve the repeated ones
+                prompts = [[random.randint(0, 30000) for _ in range(plen)] for _ in range(num)]
+                torch.cuda.synchronize()
+                llm.generate(prompts, params, use_tqdm=False)
+                torch.cuda.synchronize()
+                if i:
+                    runs.append(dict(llm.last_stats))
+            llm._exit()
+            del llm
+            torch.cuda.empty_cache()
+            agg = {k: sum(r[k] for r in runs) for k in runs[0]}
+            row[label] = {"prefill_tok_s": round(agg["prefill_tokens"] / agg["prefill_s"], 1),
+                          "decode_tok_s": round(agg["decode_tokens"] / agg["decode_s"], 1),
+                          "decode_ms_per_step": round(1e3 * agg["decode_s"] / agg["decode_steps"], 3)}
+        results.append(row)
+    print(json.dumps({"metric": "prefill and decode tokens/s, Rurutar beside the dense Qwen3 decoder at equal size",
+                      "unit": "tokens/s", "n_gpus": 1, "dtype": "bf16", "data": "synthetic (random weights, random prompts)",
+                      "higher_is_better": True, "sizes": results}), flush=True)
+
+
 KEEPER = r"""
 import os, select, signal, sys
 # a launcher that ends a failed job signals the ranks' whole process groups, this process included, possibly while
@@ -364,7 +444,14 @@ def main():
     ap.add_argument("--single-leg", action="store_true", help="tp: time only the --allreduce leg")
     ap.add_argument("--eager", action="store_true", help="no hipGraph (debug)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--arch-compare", action="store_true",
+                    help="instead of the decode benchmark: prefill and decode tokens/s of the Rurutar design beside the "
+                         "dense Qwen3 decoder at equal size (one GPU, LLM.generate)")
+    ap.add_argument("--arch-sizes", default="", help="--arch-compare: comma-separated subset of " + ",".join(ARCH_COMPARE_SIZES))
     args = ap.parse_args()
+    if args.arch_compare:
+        torch.cuda.set_device(0)
+        return run_arch_compare(args)
 
     if args.gpus > 1 and "WORLD_SIZE" not in os.environ:
         sys.exit(self_launch(args.gpus, sys.argv[1:]))

@@ -74,7 +74,7 @@ _PROTOS = {
     "nv_gla_recurrent": (_i, [_p, _i64, _i, _i, _i, _i, _p, _i64, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _f, _f, _f, _i, _p]),
     "nv_latent_kv_store": (_i, [_p, _i64, _p, _p, _p, _f, _p, _p, _i64, _i, _i, _i, _f, _i, _p]),
     "nv_latent_q_rope": (_i, [_p, _i64, _p, _p, _f, _p, _i64, _i, _i, _i, _i, _i, _i, _p]),
-    "nv_latent_attn": (_i, [_p, _p, _p, _i, _p, _p, _p, _p, _i64, _i, _i, _i, _i, _i, _f, _i, _p]),
+    "nv_latent_attn": (_i, [_p, _p, _p, _i, _p, _p, _p, _p, _i64, _i, _i, _i, _i, _i, _i, _f, _i, _p]),
     "nv_moe_route": (_i, [_p, _i64, _p, _p, _i64, _i, _i, _p]),
     "nv_moe_sort": (_i, [_p, _i64, _i, _i, _p, _p, _p, _p]),
     "nv_moe_combine": (_i, [_p, _p, _p, _i, _p, _p, _i64, _p, _i64, _i, _p]),

@@ -5,8 +5,9 @@
 // from the request's state slot (or from zero when the request has no tokens behind it) and leaving the state there:
 // a prompt portion, the next portion and single decoded tokens all go through this one kernel.
 //
-// Thread (part, v) keeps the state entries S[part + parts * i][v], i < DPT, in registers; the o_t column sums over the
-// parts go through LDS.  The decay is evaluated as exp(log(sigmoid(z)) / tau) with log(sigmoid) in its stable form.
+// Two kernels: gla_col_kernel (key sizes up to 128: one state column per thread, see there) and gla_kernel for wider
+// states, where thread (part, v) keeps the state entries S[part + parts * i][v], i < DPT, in registers and the o_t
+// column sums over the parts go through LDS.  The decay is evaluated as exp(log(sigmoid(z)) / tau) with log(sigmoid) in its stable form.
 #include "anyt.h"
 
 namespace {
@@ -90,6 +91,129 @@ __global__ __launch_bounds__(1024) void gla_kernel(GlaArgs p) {
   }
 }
 
+
+// The usual shape (dim <= 128): thread v owns the whole state column S[:, v] in registers, so o_t[v] needs no sum
+// across threads.  Tokens are staged sixteen at a time: decay, k and q rows in LDS (padded to DMAX with a = 1,
+// k = q = 0), the thread's own v and gate values in registers; the per-token loop then only reads LDS broadcasts, four
+// channels per read; the RMS norm's sum over vdim is taken for the sixteen tokens at once (three barriers per chunk).
+constexpr int GLA_TC = 16;
+
+constexpr int gla_col_threads(int dmax) { return dmax >= 64 ? 256 : 512; }   // bounded by registers per thread
+
+template <typename T, int DMAX>
+__global__ __launch_bounds__(gla_col_threads(DMAX)) void gla_col_kernel(GlaArgs p) {
+  extern __shared__ float4 lds4[];
+  float* lds = reinterpret_cast<float*>(lds4);
+  const int vd = p.vdim;
+  float* sa = lds;                       // [TC][DMAX]
+  float* sk = sa + GLA_TC * DMAX;
+  float* sq = sk + GLA_TC * DMAX;
+  float* sred = sq + GLA_TC * DMAX;      // [TC][waves]
+  const int h = blockIdx.x, b = blockIdx.y;
+  const int tid = threadIdx.x, nthr = blockDim.x, wv = tid >> 6, nw = nthr >> 6;
+  const bool active = tid < vd;
+  const int col = active ? tid : 0;
+  const int t0 = p.cu_q[b], t1 = p.cu_q[b + 1];
+  if (t1 <= t0) return;
+  float* S_g = p.state + ((int64_t)p.slots[b] * p.H + h) * p.dim * vd;
+  float S[DMAX];
+  const bool fresh = p.past[b] == 0;
+#pragma unroll
+  for (int i = 0; i < DMAX; ++i) S[i] = (active && i < p.dim && !fresh) ? S_g[(int64_t)i * vd + tid] : 0.0f;
+  const float nw_v = active ? ld_f32<T>(reinterpret_cast<const T*>(p.norm_w) + tid) : 0.0f;
+  for (int c0 = t0; c0 < t1; c0 += GLA_TC) {
+    const int nt = min(GLA_TC, t1 - c0);
+    // this thread's own v and gate values of the chunk: sixteen loads in flight, no LDS
+    float vreg[GLA_TC], greg[GLA_TC];
+#pragma unroll
+    for (int j = 0; j < GLA_TC; ++j) {
+      vreg[j] = greg[j] = 0.0f;
+      if (j < nt) {
+        const float* row = p.proj + (int64_t)(c0 + j) * p.proj_rs;
+        vreg[j] = row[p.v_off + h * vd + col];
+        greg[j] = row[p.g_off + h * vd + col];
+      }
+    }
+    __syncthreads();                     // the previous chunk's rows are no longer read
+    // decay, k and q rows of the chunk, four elements per thread and round so that the loads overlap
+    for (int base = tid * 4; base < nt * DMAX; base += nthr * 4) {
+      const int j = base / DMAX, i = base % DMAX;          // DMAX is a multiple of 4: the four share a token
+      float z4[4], k4[4], q4[4];
+      const bool live = j < nt;
+      const float* row = p.proj + (int64_t)(c0 + (live ? j : 0)) * p.proj_rs;
+      const float* zr = p.z + (int64_t)(c0 + (live ? j : 0)) * p.z_rs;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const bool in = live && i + e < p.dim;
+        const int ch = h * p.dim + (in ? i + e : 0);
+        z4[e] = zr[ch];
+        k4[e] = in ? row[p.k_off + ch] : 0.0f;
+        q4[e] = in ? row[p.q_off + ch] * p.q_scale : 0.0f;
+        z4[e] = in ? expf(log_sigmoid_f32(z4[e]) * p.inv_tau) : 1.0f;
+      }
+      *reinterpret_cast<float4*>(sa + base) = make_float4(z4[0], z4[1], z4[2], z4[3]);
+      *reinterpret_cast<float4*>(sk + base) = make_float4(k4[0], k4[1], k4[2], k4[3]);
+      *reinterpret_cast<float4*>(sq + base) = make_float4(q4[0], q4[1], q4[2], q4[3]);
+    }
+    __syncthreads();
+    float o[GLA_TC];
+#pragma unroll
+    for (int j = 0; j < GLA_TC; ++j) {
+      float acc0 = 0.0f, acc1 = 0.0f;
+      if (j < nt) {
+        const float vv = vreg[j];
+        const float4* a4 = reinterpret_cast<const float4*>(sa + j * DMAX);
+        const float4* k4 = reinterpret_cast<const float4*>(sk + j * DMAX);
+        const float4* q4 = reinterpret_cast<const float4*>(sq + j * DMAX);
+#pragma unroll
+        for (int i = 0; i < DMAX / 4; ++i) {
+          const float4 a = a4[i], k = k4[i], q = q4[i];
+          S[4 * i + 0] = a.x * S[4 * i + 0] + k.x * vv;
+          S[4 * i + 1] = a.y * S[4 * i + 1] + k.y * vv;
+          S[4 * i + 2] = a.z * S[4 * i + 2] + k.z * vv;
+          S[4 * i + 3] = a.w * S[4 * i + 3] + k.w * vv;
+          acc0 += S[4 * i + 0] * q.x;
+          acc1 += S[4 * i + 1] * q.y;
+          acc0 += S[4 * i + 2] * q.z;
+          acc1 += S[4 * i + 3] * q.w;
+        }
+      }
+      o[j] = acc0 + acc1;
+      const float ss = wave_sum(active ? o[j] * o[j] : 0.0f);
+      if ((tid & 63) == 0) sred[j * nw + wv] = ss;
+    }
+    __syncthreads();
+    if (active) {
+#pragma unroll
+      for (int j = 0; j < GLA_TC; ++j) {
+        if (j < nt) {
+          float ss = 0.0f;
+          for (int w = 0; w < nw; ++w) ss += sred[j * nw + w];
+          const float inv = 1.0f / sqrtf(ss / (float)vd + p.eps);
+          st_f32<T>(reinterpret_cast<T*>(p.out) + (int64_t)(c0 + j) * p.H * vd + h * vd + tid,
+                    o[j] * inv * nw_v * silu_f32(greg[j]));
+        }
+      }
+    }
+  }
+  if (active) {
+#pragma unroll
+    for (int i = 0; i < DMAX; ++i)
+      if (i < p.dim) S_g[(int64_t)i * vd + tid] = S[i];
+  }
+}
+
+template <typename T>
+int launch_col(const GlaArgs& p, int dmax, dim3 grid, int threads, size_t lds, hipStream_t s) {
+  switch (dmax) {
+    case 16: gla_col_kernel<T, 16><<<grid, dim3(threads), lds, s>>>(p); break;
+    case 32: gla_col_kernel<T, 32><<<grid, dim3(threads), lds, s>>>(p); break;
+    case 64: gla_col_kernel<T, 64><<<grid, dim3(threads), lds, s>>>(p); break;
+    default: gla_col_kernel<T, 128><<<grid, dim3(threads), lds, s>>>(p); break;
+  }
+  return 0;
+}
+
 template <typename T>
 int launch(const GlaArgs& p, int dpt, dim3 grid, int threads, size_t lds, hipStream_t s) {
   switch (dpt) {
@@ -114,6 +238,19 @@ extern "C" int nv_gla_recurrent(const float* proj, int64_t proj_row_stride, int 
                "nv_gla_recurrent: bad shape heads=%d dim=%d vdim=%d seqs=%d", heads, dim, vdim, num_seqs);
   NV_CHECK_ARG(tau > 0.0f, "nv_gla_recurrent: tau must be positive");
   if (num_seqs == 0) return NV_OK;
+  if (dim <= 128) {     // one state column per thread
+    int dmax = 16;
+    while (dmax < dim) dmax *= 2;
+    const int threads = ((vdim + 63) / 64) * 64;
+    const size_t lds = (size_t)(GLA_TC * 3 * dmax + GLA_TC * (threads / 64)) * sizeof(float);
+    if (lds <= 64 * 1024 && threads <= gla_col_threads(dmax)) {
+      GlaArgs p{proj, proj_row_stride, q_off, k_off, v_off, g_off, z, z_row_stride, state, cu_q, past_lens, state_slots,
+                norm_w, out, heads, dim, vdim, 1, 1.0f / tau, q_scale, eps};
+      NV_DISPATCH_T(dtype, launch_col<T>(p, dmax, dim3(heads, num_seqs), threads, lds, (hipStream_t)stream));
+      NV_CHECK_LAUNCH();
+      return NV_OK;
+    }
+  }
   int dpt = 8;
   while (dpt <= 64 && ((dim + dpt - 1) / dpt) * vdim > 1024) dpt *= 2;
   if (dpt > 64) {

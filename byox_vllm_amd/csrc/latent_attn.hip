@@ -173,6 +173,197 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(AttnArgs p) {
   }
 }
 
+
+// ---- the same attention on the matrix cores (bf16 cache) ----
+// A workgroup owns 16 query rows: TQ consecutive tokens of one request times HQ heads (HQ * TQ = 16), which all read
+// the same key rows.  Per tile of 64 keys: the rows are staged in LDS twice (row-major for S = Q K^T, transposed for
+// O += P V), wavefront w computes the scores of keys 16 w .. 16 w + 15, the softmax statistics are updated by
+// 16 threads per row, and every wavefront accumulates its share of the output columns.  Scores, maxima, sums and the
+// rescaling are fp32.  Queries and softmax weights enter the MFMAs as the sum of two bf16 numbers (value = hi + lo,
+// two MFMAs), so neither is rounded to 8 bits of mantissa; the cached rows are bf16 as stored.
+constexpr int ATT_KEYS = 64, ATT_PST = 72, ATT_SST = 68;
+
+struct MfmaAttnArgs {
+  AttnArgs a;
+  int B, HQ, TQ, Dkp;
+};
+
+template <int NTILE>
+__global__ __launch_bounds__(256) void latent_attn_mfma_kernel(MfmaAttnArgs q) {
+  extern __shared__ u32x4 lds_raw[];
+  const AttnArgs& p = q.a;
+  const int Dk = p.rank + p.rot_dim, R = p.rank, Dq = q.Dkp + 8;
+  bf16_t* sQhi = reinterpret_cast<bf16_t*>(lds_raw);
+  bf16_t* sQlo = sQhi + 16 * Dq;
+  bf16_t* sK = sQlo + 16 * Dq;
+  bf16_t* sVt = sK + ATT_KEYS * Dq;
+  bf16_t* sPhi = sVt + R * ATT_PST;
+  bf16_t* sPlo = sPhi + 16 * ATT_PST;
+  float* sS = reinterpret_cast<float*>(sPlo + 16 * ATT_PST);
+  float* sm = sS + 16 * ATT_SST;
+  float* sl = sm + 16;
+  float* scorr = sl + 16;
+  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6, c = lane & 15, g = lane >> 4;
+
+  // which request and which of its tokens this tile covers
+  int b = 0, before = 0, tstart = 0, tcount = 0;
+  for (; b < q.B; ++b) {
+    const int len = p.cu_q[b + 1] - p.cu_q[b];
+    const int tiles = (len + q.TQ - 1) / q.TQ;
+    if ((int)blockIdx.y < before + tiles) {
+      tstart = p.cu_q[b] + ((int)blockIdx.y - before) * q.TQ;
+      tcount = min(q.TQ, p.cu_q[b + 1] - tstart);
+      break;
+    }
+    before += tiles;
+  }
+  if (b == q.B) return;
+  const int h0 = blockIdx.x * q.HQ;
+  const int pos0 = p.past[b] + (tstart - p.cu_q[b]);
+  const int kmax = pos0 + tcount - 1;
+  const int kmin = p.window > 0 ? max(0, pos0 - p.window + 1) : 0;
+  const int32_t* table = p.tables + (int64_t)b * p.table_cols;
+  const bf16_t* cache = reinterpret_cast<const bf16_t*>(p.cache);
+
+  for (int i = tid; i < ATT_KEYS * Dq; i += 256) sK[i] = (bf16_t)0.0f;       // the padding columns stay zero
+  for (int i = tid; i < 16 * Dq; i += 256) {
+    const int r = i / Dq, f = i % Dq;
+    const int tq = r / q.HQ, hh = h0 + r % q.HQ;
+    float v = 0.0f;
+    if (tq < tcount && hh < p.H && f < Dk) v = p.qa[((int64_t)(tstart + tq) * p.H + hh) * Dk + f];
+    const bf16_t hi = (bf16_t)v;
+    sQhi[i] = hi;
+    sQlo[i] = (bf16_t)(v - (float)hi);
+  }
+  if (tid < 16) {
+    sm[tid] = -INFINITY;
+    sl[tid] = 0.0f;
+  }
+  f32x4 O[NTILE];
+#pragma unroll
+  for (int n = 0; n < NTILE; ++n) O[n] = f32x4{0.f, 0.f, 0.f, 0.f};
+  // the row this thread serves in the softmax step
+  const int srow = tid >> 4, skq = tid & 15;
+  const int s_tq = srow / q.HQ, s_hh = h0 + srow % q.HQ;
+  const bool s_valid = s_tq < tcount && s_hh < p.H;
+  const int s_pos = pos0 + s_tq;
+  const int s_lo = p.window > 0 ? max(0, s_pos - p.window + 1) : 0;
+  const int chunks = Dk / 8;
+  __syncthreads();
+
+  for (int j0 = kmin; j0 <= kmax; j0 += ATT_KEYS) {
+    // stage the key rows: consecutive threads take consecutive keys (conflict-free transposed stores)
+    for (int i = tid; i < ATT_KEYS * chunks; i += 256) {
+      const int key = i % ATT_KEYS, f8 = i / ATT_KEYS;
+      const int kp = j0 + key;
+      u32x4 v = u32x4{0u, 0u, 0u, 0u};
+      if (kp <= kmax) {
+        const int64_t row = (int64_t)table[kp / p.block_size] * p.block_size + kp % p.block_size;
+        v = *reinterpret_cast<const u32x4*>(cache + row * Dk + f8 * 8);
+      }
+      *reinterpret_cast<u32x4*>(sK + key * Dq + f8 * 8) = v;
+      if (f8 * 8 < R) {
+        const uint16_t* e16 = reinterpret_cast<const uint16_t*>(&v);
+        uint16_t* dst = reinterpret_cast<uint16_t*>(sVt) + (f8 * 8) * ATT_PST + key;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) dst[e * ATT_PST] = e16[e];
+      }
+    }
+    __syncthreads();
+    // S = Q K^T for this wavefront's 16 keys
+    {
+      f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+      const bf16_t* krow = sK + (16 * wv + c) * Dq + 8 * g;
+      const bf16_t* qhi = sQhi + c * Dq + 8 * g;
+      const bf16_t* qlo = sQlo + c * Dq + 8 * g;
+      for (int ks = 0; ks < q.Dkp; ks += 32) {
+        const bf16x8 kf = *reinterpret_cast<const bf16x8*>(krow + ks);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<const bf16x8*>(qhi + ks), kf, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<const bf16x8*>(qlo + ks), kf, acc, 0, 0, 0);
+      }
+#pragma unroll
+      for (int r = 0; r < 4; ++r) sS[(4 * g + r) * ATT_SST + 16 * wv + c] = acc[r] * p.scale;
+    }
+    __syncthreads();
+    // softmax statistics: 16 threads per row, 4 keys each
+    {
+      float sv[4], m = -INFINITY;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int kp = j0 + 4 * skq + e;
+        const bool ok = s_valid && kp >= s_lo && kp <= s_pos;
+        sv[e] = ok ? sS[srow * ATT_SST + 4 * skq + e] : -INFINITY;
+        m = fmaxf(m, sv[e]);
+      }
+#pragma unroll
+      for (int o = 8; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+      const float m_old = sm[srow];
+      const float m_new = fmaxf(m_old, m);
+      float sum = 0.0f;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float pe = (sv[e] == -INFINITY) ? 0.0f : expf(sv[e] - m_new);
+        sum += pe;
+        const bf16_t hi = (bf16_t)pe;
+        sPhi[srow * ATT_PST + 4 * skq + e] = hi;
+        sPlo[srow * ATT_PST + 4 * skq + e] = (bf16_t)(pe - (float)hi);
+      }
+#pragma unroll
+      for (int o = 8; o > 0; o >>= 1) sum += __shfl_xor(sum, o, 64);
+      if (skq == 0) {
+        const float corr = (m_new == -INFINITY) ? 1.0f : expf(m_old - m_new);
+        scorr[srow] = corr;
+        sm[srow] = m_new;
+        sl[srow] = sl[srow] * corr + sum;
+      }
+    }
+    __syncthreads();
+    // O = O * corr + P V for this wavefront's output columns
+#pragma unroll
+    for (int n = 0; n < NTILE; ++n) {
+      const int col0 = 16 * (wv * NTILE + n);
+      if (col0 < R) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) O[n][r] *= scorr[4 * g + r];
+#pragma unroll
+        for (int ks = 0; ks < ATT_KEYS; ks += 32) {
+          const bf16x8 vf = *reinterpret_cast<const bf16x8*>(sVt + (col0 + c) * ATT_PST + ks + 8 * g);
+          O[n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+              *reinterpret_cast<const bf16x8*>(sPhi + c * ATT_PST + ks + 8 * g), vf, O[n], 0, 0, 0);
+          O[n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+              *reinterpret_cast<const bf16x8*>(sPlo + c * ATT_PST + ks + 8 * g), vf, O[n], 0, 0, 0);
+        }
+      }
+    }
+    __syncthreads();
+  }
+  bf16_t* out = reinterpret_cast<bf16_t*>(p.out);
+#pragma unroll
+  for (int n = 0; n < NTILE; ++n) {
+    const int col = 16 * (wv * NTILE + n) + c;
+    if (col >= R) continue;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int row = 4 * g + r;
+      const int tq = row / q.HQ, hh = h0 + row % q.HQ;
+      if (tq < tcount && hh < p.H) out[((int64_t)(tstart + tq) * p.H + hh) * R + col] = (bf16_t)(O[n][r] / sl[row]);
+    }
+  }
+}
+
+template <int NTILE>
+hipError_t launch_mfma_attn(const MfmaAttnArgs& q, dim3 grid, size_t lds, hipStream_t s) {
+  static size_t allowed = 64 * 1024;
+  if (lds > allowed) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&latent_attn_mfma_kernel<NTILE>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return e;
+    allowed = lds;
+  }
+  latent_attn_mfma_kernel<NTILE><<<grid, dim3(256), lds, s>>>(q);
+  return hipSuccess;
+}
+
 }  // namespace
 
 extern "C" int nv_latent_kv_store(const float* kv, int64_t kv_row_stride, const void* norm_w, const int64_t* positions,
@@ -207,7 +398,7 @@ extern "C" int nv_latent_q_rope(const void* q, int64_t q_row_stride, const int64
 
 extern "C" int nv_latent_attn(const float* qa, const void* cache, const int32_t* block_tables, int table_cols,
                               const int32_t* cu_q, const int32_t* past_lens, const int32_t* seq_of_token, void* out,
-                              int64_t tokens, int heads, int rank, int rot_dim, int block_size, int window, float scale,
+                              int64_t tokens, int num_seqs, int heads, int rank, int rot_dim, int block_size, int window, float scale,
                               int dtype, nv_stream_t stream) {
   NV_CHECK_ARG(qa && cache && block_tables && cu_q && past_lens && seq_of_token && out, "nv_latent_attn: null pointer");
   NV_CHECK_ARG(dtype == NV_BF16 || dtype == NV_F32, "nv_latent_attn: bad dtype %d", dtype);
@@ -216,6 +407,32 @@ extern "C" int nv_latent_attn(const float* qa, const void* cache, const int32_t*
   if (tokens == 0) return NV_OK;
   NV_CHECK_ARG(tokens <= 65535, "nv_latent_attn: %lld tokens exceed one launch", (long long)tokens);
   const int Dk = rank + rot_dim;
+  // bf16 caches whose rows split into 16-byte pieces go to the matrix cores
+  if (dtype == NV_BF16 && Dk % 8 == 0 && rank % 16 == 0 && rank <= 512 && num_seqs > 0) {
+    int HQ = 1;
+    while (HQ < heads && HQ < 16) HQ *= 2;
+    MfmaAttnArgs q{{qa, cache, block_tables, table_cols, cu_q, past_lens, seq_of_token, out, heads, rank, rot_dim,
+                    block_size, window, 0, 0, scale},
+                   num_seqs, HQ, 16 / HQ, ((Dk + 31) / 32) * 32};
+    const int Dq = q.Dkp + 8;
+    const size_t lds = (size_t)(2 * 16 * Dq + ATT_KEYS * Dq + rank * ATT_PST + 2 * 16 * ATT_PST) * 2 +
+                       (size_t)(16 * ATT_SST + 48) * 4;
+    if (lds <= 150 * 1024) {
+      const int64_t tiles = tokens / q.TQ + num_seqs;        // at most: every request may end in a partial tile
+      NV_CHECK_ARG(tiles <= 65535, "nv_latent_attn: %lld tiles exceed one launch", (long long)tiles);
+      dim3 grid((unsigned)((heads + HQ - 1) / HQ), (unsigned)tiles);
+      const int ntile = (rank / 16 + 3) / 4;
+      hipError_t e = ntile <= 2   ? launch_mfma_attn<2>(q, grid, lds, (hipStream_t)stream)
+                     : ntile <= 4 ? launch_mfma_attn<4>(q, grid, lds, (hipStream_t)stream)
+                                  : launch_mfma_attn<8>(q, grid, lds, (hipStream_t)stream);
+      if (e != hipSuccess) {
+        nv_set_error("nv_latent_attn: %s", hipGetErrorString(e));
+        return NV_ERR_LAUNCH;
+      }
+      NV_CHECK_LAUNCH();
+      return NV_OK;
+    }
+  }
   // LDS plan: as many heads per workgroup as fit beside a key tile of 64 (then 32, 16, 8) rows
   const size_t budget = 64 * 1024;
   int TK = 64, HC = heads;

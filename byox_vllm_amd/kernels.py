@@ -578,7 +578,8 @@ def latent_attn(qa, cache, block_tables, cu_q, past_lens, seq_of_token, heads, r
     assert cu_q.dtype == past_lens.dtype == seq_of_token.dtype == torch.int32 and seq_of_token.numel() == T
     out = torch.empty(T, heads * rank, dtype=cache.dtype, device=qa.device) if out is None else out
     check(lib().nv_latent_attn(ptr(qa), ptr(cache), ptr(block_tables), block_tables.size(1), ptr(cu_q), ptr(past_lens),
-                               ptr(seq_of_token), ptr(out), T, heads, rank, rot_dim, block_size, window, scale,
+                               ptr(seq_of_token), ptr(out), T, past_lens.numel(), heads, rank, rot_dim, block_size, window,
+                               scale,
                                _code32(cache.dtype), stream()), "nv_latent_attn")
     return out
 

@@ -376,7 +376,8 @@ int nv_latent_q_rope(const void* q, int64_t q_row_stride, const int64_t* positio
                      float* qa, int64_t tokens, int heads, int dim, int rot_dim, int rot_dims, int rank, int dtype,
                      nv_stream_t stream);
 int nv_latent_attn(const float* qa, const void* cache, const int32_t* block_tables, int table_cols, const int32_t* cu_q,
-                   const int32_t* past_lens, const int32_t* seq_of_token, void* out, int64_t tokens, int heads, int rank,
+                   const int32_t* past_lens, const int32_t* seq_of_token, void* out, int64_t tokens, int num_seqs, int heads,
+                   int rank,
                    int rot_dim, int block_size, int window, float scale, int dtype, nv_stream_t stream);
 
 /* Mixture of experts (csrc/moe.hip): routing, ordering by expert, weighted combination. */

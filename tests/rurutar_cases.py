@@ -60,6 +60,16 @@ def odd_config():
     ], softcap=None, scale=1.0)
 
 
+def aligned_config():
+    """Sizes in multiples of 16 and 32, where the 16-bit engine takes its matrix-core kernels; dense feed-forwards only,
+    so that 16-bit runs have no routing decisions to flip."""
+    return config(256, 128, [
+        (latent(6, 16, 8, 16, 32, 24, window=11, scaling=SCALING), dense(96)),
+        (gla(2, 32, 64, 6.0), dense(64)),
+        (latent(3, 32, 8, 32, 32, 48, window=40, scaling=SCALING, kv_from=0), None),
+    ], softcap=15.0)
+
+
 def engine_config(cfg_json, weights, dtype, blocks=16, slots=4, block_size=16, decay_rank=None, **kw):
     """The engine's Config for an in-memory checkpoint of one of the configurations above."""
     from byox_vllm_amd.config import Config
