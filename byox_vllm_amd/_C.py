@@ -40,6 +40,7 @@ _PROTOS = {
     "nv_silu_mul": (_i, [_p, _p, _i64, _i, _i, _p]),
     "nv_gemm_lt_available": (_i, []),
     "nv_gemm_lt": (_i, [_p, _i64, _p, _p, _p, _i64, _i, _i, _i, _i, _p, _sz, _p]),
+    "nv_gemm_lt_f32out": (_i, [_p, _i64, _p, _p, _i64, _i, _i, _i, _i, _p, _sz, _p]),
     "nv_weight_expand": (_i, [_p, _p, _i, _i, _i, _i, _i, _p, _p]),
     "nv_gemm_workspace_bytes": (_sz, [_i64, _i, _i]),
     "nv_gemm_pick_split_k": (_i, [_i64, _i, _i, _i]),
@@ -70,6 +71,7 @@ _PROTOS = {
     "nv_embed_scale": (_i, [_p, _p, _p, _i64, _i, _i64, _f, _i, _p]),
     "nv_dyt_norm": (_i, [_p, _p, _i64, _p, _p, _p, _p, _p, _i64, _i, _i, _p]),
     "nv_rmsnorm_f32": (_i, [_p, _i64, _p, _p, _i64, _i64, _i, _f, _i, _p]),
+    "nv_act_mul_f32": (_i, [_p, _p, _i64, _i, _i, _i, _p]),
     "nv_sample_f32": (_i, [_p, _i64, _p, _p, _i, _i, _u64, _p]),
     "nv_gla_recurrent": (_i, [_p, _i64, _i, _i, _i, _i, _p, _i64, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _f, _f, _f, _i, _p]),
     "nv_latent_kv_store": (_i, [_p, _i64, _p, _p, _p, _f, _p, _p, _i64, _i, _i, _i, _f, _i, _p]),

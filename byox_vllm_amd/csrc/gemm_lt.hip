@@ -96,15 +96,34 @@ void destroy_plan(LtApi& api, LtPlan& p) {
 
 extern "C" int nv_gemm_lt_available(void) { return lt_api().ok ? 1 : 0; }
 
+static int gemm_lt_impl(const void* x, int64_t x_row_stride, const void* w_rowmajor, const void* bias, void* out,
+                        int64_t out_row_stride, int M, int N, int K, int dtype, void* workspace, size_t workspace_bytes,
+                        nv_stream_t stream, int out_f32);
+
 extern "C" int nv_gemm_lt(const void* x, int64_t x_row_stride, const void* w_rowmajor, const void* bias, void* out,
                           int64_t out_row_stride, int M, int N, int K, int dtype, void* workspace,
                           size_t workspace_bytes, nv_stream_t stream) {
+  return gemm_lt_impl(x, x_row_stride, w_rowmajor, bias, out, out_row_stride, M, N, K, dtype, workspace, workspace_bytes,
+                      stream, 0);
+}
+
+// the same product written as fp32 rows (16-bit operands, fp32 accumulation, no rounding of the result)
+extern "C" int nv_gemm_lt_f32out(const void* x, int64_t x_row_stride, const void* w_rowmajor, float* out,
+                                 int64_t out_row_stride, int M, int N, int K, int dtype, void* workspace,
+                                 size_t workspace_bytes, nv_stream_t stream) {
+  return gemm_lt_impl(x, x_row_stride, w_rowmajor, nullptr, out, out_row_stride, M, N, K, dtype, workspace,
+                      workspace_bytes, stream, 1);
+}
+
+static int gemm_lt_impl(const void* x, int64_t x_row_stride, const void* w_rowmajor, const void* bias, void* out,
+                        int64_t out_row_stride, int M, int N, int K, int dtype, void* workspace, size_t workspace_bytes,
+                        nv_stream_t stream, int out_f32) {
   NV_CHECK_ARG(x && w_rowmajor && out, "nv_gemm_lt: null pointer");
   NV_CHECK_ARG(dtype == NV_BF16 || dtype == NV_F16, "nv_gemm_lt: bad dtype %d", dtype);
   NV_CHECK_ARG(M > 0 && N > 0 && K > 0 && x_row_stride >= K && out_row_stride >= N, "nv_gemm_lt: M=%d N=%d K=%d strides %lld %lld",
                M, N, K, (long long)x_row_stride, (long long)out_row_stride);
   NV_CHECK_ARG(((uintptr_t)x | (uintptr_t)w_rowmajor | (uintptr_t)out | (uintptr_t)workspace) % 16 == 0 && K % 8 == 0 &&
-                   N % 8 == 0 && x_row_stride % 8 == 0 && out_row_stride % 8 == 0,
+                   N % 8 == 0 && x_row_stride % 8 == 0 && out_row_stride % (out_f32 ? 4 : 8) == 0,
                "nv_gemm_lt: operands must be 16-byte aligned (K, N and the row strides multiples of 8)");
   LtApi& api = lt_api();
   NV_CHECK_ARG(api.ok, "nv_gemm_lt: %s", api.why);
@@ -120,7 +139,7 @@ extern "C" int nv_gemm_lt(const void* x, int64_t x_row_stride, const void* w_row
     nv_set_error("nv_gemm_lt: hipblasLtCreate failed");
     return NV_ERR_LAUNCH;
   }
-  const LtKey key(device, M, N, K, dtype, bias ? 1 : 0, x_row_stride, out_row_stride, workspace_bytes);
+  const LtKey key(device, M, N, K, dtype, (bias ? 1 : 0) | (out_f32 ? 2 : 0), x_row_stride, out_row_stride, workspace_bytes);
   auto it = g_lt_plans.find(key);
   if (it == g_lt_plans.end()) {
     // Row-major out[M, N] = x[M, K] * W[N, K]^T is, read column-major, D (N x M) = W^T-as-stored (K x N, transposed)
@@ -139,7 +158,7 @@ extern "C" int nv_gemm_lt(const void* x, int64_t x_row_stride, const void* w_row
     }
     ok = ok && api.LayoutCreate(&p.a, t, (uint64_t)K, (uint64_t)N, (int64_t)K) == HIPBLAS_STATUS_SUCCESS;
     ok = ok && api.LayoutCreate(&p.b, t, (uint64_t)K, (uint64_t)M, x_row_stride) == HIPBLAS_STATUS_SUCCESS;
-    ok = ok && api.LayoutCreate(&p.c, t, (uint64_t)N, (uint64_t)M, out_row_stride) == HIPBLAS_STATUS_SUCCESS;
+    ok = ok && api.LayoutCreate(&p.c, out_f32 ? HIP_R_32F : t, (uint64_t)N, (uint64_t)M, out_row_stride) == HIPBLAS_STATUS_SUCCESS;
     if (!ok) {
       destroy_plan(api, p);
       nv_set_error("nv_gemm_lt: descriptor set-up failed (M=%d N=%d K=%d)", M, N, K);

@@ -252,21 +252,33 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(MfmaAttnArgs q) {
   __syncthreads();
 
   for (int j0 = kmin; j0 <= kmax; j0 += ATT_KEYS) {
-    // stage the key rows: consecutive threads take consecutive keys (conflict-free transposed stores)
-    for (int i = tid; i < ATT_KEYS * chunks; i += 256) {
-      const int key = i % ATT_KEYS, f8 = i / ATT_KEYS;
-      const int kp = j0 + key;
-      u32x4 v = u32x4{0u, 0u, 0u, 0u};
-      if (kp <= kmax) {
-        const int64_t row = (int64_t)table[kp / p.block_size] * p.block_size + kp % p.block_size;
-        v = *reinterpret_cast<const u32x4*>(cache + row * Dk + f8 * 8);
-      }
-      *reinterpret_cast<u32x4*>(sK + key * Dq + f8 * 8) = v;
-      if (f8 * 8 < R) {
-        const uint16_t* e16 = reinterpret_cast<const uint16_t*>(&v);
-        uint16_t* dst = reinterpret_cast<uint16_t*>(sVt) + (f8 * 8) * ATT_PST + key;
+    // stage the key rows: consecutive threads take consecutive keys (conflict-free transposed stores); four loads are
+    // issued before the first is stored, so their latencies overlap
+    for (int i0 = tid; i0 < ATT_KEYS * chunks; i0 += 4 * 256) {
+      u32x4 v[4];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) dst[e * ATT_PST] = e16[e];
+      for (int u = 0; u < 4; ++u) {
+        const int i = i0 + u * 256;
+        const int key = i % ATT_KEYS, f8 = i / ATT_KEYS;
+        const int kp = j0 + key;
+        v[u] = u32x4{0u, 0u, 0u, 0u};
+        if (f8 < chunks && kp <= kmax) {
+          const int64_t row = (int64_t)table[kp / p.block_size] * p.block_size + kp % p.block_size;
+          v[u] = *reinterpret_cast<const u32x4*>(cache + row * Dk + f8 * 8);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int i = i0 + u * 256;
+        const int key = i % ATT_KEYS, f8 = i / ATT_KEYS;
+        if (f8 >= chunks) continue;
+        *reinterpret_cast<u32x4*>(sK + key * Dq + f8 * 8) = v[u];
+        if (f8 * 8 < R) {
+          const uint16_t* e16 = reinterpret_cast<const uint16_t*>(&v[u]);
+          uint16_t* dst = reinterpret_cast<uint16_t*>(sVt) + (f8 * 8) * ATT_PST + key;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) dst[e * ATT_PST] = e16[e];
+        }
       }
     }
     __syncthreads();

@@ -51,6 +51,18 @@ __global__ __launch_bounds__(256) void rmsnorm_f32_kernel(const float* __restric
   for (int j = threadIdx.x; j < n; j += blockDim.x) st_f32<T>(out + r * out_rs + j, xr[j] * inv * ld_f32<T>(w + j));
 }
 
+// out[m][j] = act(y[m][j]) * y[m][n + j]: the gated unit's activation over a plain product's [gate | up] rows
+template <typename T>
+__global__ __launch_bounds__(256) void act_mul_f32_kernel(const float* __restrict__ y, T* __restrict__ out, int64_t total,
+                                                          int n, int act) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t m = i / n;
+    const int j = (int)(i - m * n);
+    const float g = y[m * 2 * n + j], u = y[m * 2 * n + n + j];
+    st_f32<T>(out + i, (act == 1 ? gelu_tanh_f32(g) : silu_f32(g)) * u);
+  }
+}
+
 // Gumbel-max sampling from fp32 logits: argmax_j (l_j / T + g_j) with g_j = -log(-log(u_j)), u_j a hash of (seed, row,
 // column); temperature 0 takes the plain argmax.  Ties go to the lowest index.
 __device__ __forceinline__ uint32_t mix32(uint64_t x) {
@@ -110,6 +122,20 @@ extern "C" int nv_sample_f32(const float* logits, int64_t row_stride, const floa
   if (B == 0) return NV_OK;
   sample_f32_kernel<<<dim3((unsigned)B), dim3(256), 0, (hipStream_t)stream>>>(logits, row_stride, temperatures, tokens, V,
                                                                               seed);
+  NV_CHECK_LAUNCH();
+  return NV_OK;
+}
+
+extern "C" int nv_act_mul_f32(const float* y, void* out, int64_t rows, int n, int act, int dtype, nv_stream_t stream) {
+  NV_CHECK_ARG(y && out, "nv_act_mul_f32: null pointer");
+  NV_CHECK_ARG(dtype == NV_BF16 || dtype == NV_F32, "nv_act_mul_f32: bad dtype %d", dtype);
+  NV_CHECK_ARG(rows >= 0 && n > 0 && (act == 0 || act == 1), "nv_act_mul_f32: bad shape or activation");
+  if (rows == 0) return NV_OK;
+  const int64_t total = rows * n;
+  int64_t blocks = (total + 255) / 256;
+  if (blocks > 8192) blocks = 8192;
+  NV_DISPATCH_T(dtype, act_mul_f32_kernel<T><<<dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream>>>(
+                           y, (T*)out, total, n, act));
   NV_CHECK_LAUNCH();
   return NV_OK;
 }

@@ -112,8 +112,9 @@ class ModelRunner:
             if self.portioned:
                 # models that step through run_portions: pages and state slots from the layers' own specs, eager steps
                 assert self.world_size == 1, "portioned models run on one rank"
-                self.enforce_eager = True
                 self._allocate_pools()
+                if not self.enforce_eager:
+                    self._capture_portion_graphs()
             else:
                 self._warmup_model()
                 self._allocate_kv_cache()
@@ -537,9 +538,84 @@ class ModelRunner:
         for m in pages:
             m.cache = torch.zeros(rows, m.page_spec()["width"], dtype=dtype, device=self.device)
             m.block_size = self.block_size
-        for m in states:
-            m.state = torch.zeros(slots, *m.state_spec()["shape"], dtype=torch.float32, device=self.device)
+        for m in states:       # one slot more than requests: the rows that pad a captured decode batch write there
+            m.state = torch.zeros(slots + 1, *m.state_spec()["shape"], dtype=torch.float32, device=self.device)
         self.num_state_slots = slots
+
+    @torch.inference_mode()
+    def _capture_portion_graphs(self) -> None:
+        """Decode steps of a portioned model (every request brings one token) as hipGraphs, one per padded batch size,
+        sharing a pool: forward, final norm and head.  The step's integers travel as ONE pinned buffer copied into a
+        device buffer the captured kernels read through fixed views; rows that pad the batch carry slot -1 (no cache
+        row is written), read block 0 and use the spare state slot.  Sampling follows outside the graph (its seed
+        advances per call)."""
+        config, dev = self.config, self.device
+        max_bs = min(config.max_num_seqs, MAX_GRAPH_BS)
+        self.graph_bs = sorted(config.graph_batch_sizes) if config.graph_batch_sizes else graph_batch_sizes(max_bs)
+        max_bs = self.graph_bs[-1]
+        cols = max(1, min(-(-config.max_model_len // self.block_size), config.num_kvcache_blocks))
+        # words: ids (int64) | positions (int64) | slot_mapping | past_lens | state_slots | block tables
+        words = max_bs * (7 + cols)
+        self._pstage_host = torch.zeros(words, dtype=torch.int32, device="cpu").pin_memory()
+        self._pstage_np = self._pstage_host.numpy()
+        self._pstage_dev = torch.zeros(words, dtype=torch.int32, device=dev)
+        self._pstage_cols = cols
+        # 0, 1, 2, ...: token ranges, token owners and logit rows of a step with one token per request.  Kept on the
+        # runner: the captured kernels read it at every replay
+        ramp = self._pgraph_ramp = torch.arange(max_bs + 1, dtype=torch.int32, device=dev)
+        self.graphs, self.graph_pool, self._pgraph_out = {}, None, {}
+
+        def views(bs, buf):
+            at = [0, 2 * bs, 4 * bs, 5 * bs, 6 * bs, 7 * bs]
+            return dict(ids=buf[at[0]:at[1]].view(torch.int64), pos=buf[at[1]:at[2]].view(torch.int64),
+                        slots=buf[at[2]:at[3]], past=buf[at[3]:at[4]], states=buf[at[4]:at[5]],
+                        tables=buf[at[5]:at[5] + bs * cols].view(bs, cols))
+        self._pstage_views = views
+
+        def forward(bs):
+            v = views(bs, self._pstage_dev)
+            set_context(True, cu_seqlens_q=ramp[:bs + 1], max_seqlen_q=1, slot_mapping=v["slots"], block_tables=v["tables"],
+                        past_lens=v["past"], state_slots=v["states"], seq_of_token=ramp[:bs])
+            state = self.model(v["ids"], v["pos"])
+            return self.model.compute_logits(state, ramp[:bs], out_dtype=torch.float32)
+
+        for bs in reversed(self.graph_bs):
+            h = views(bs, self._pstage_host)
+            h["slots"].fill_(-1)
+            h["states"].fill_(self.num_state_slots)
+            self._pstage_dev[:bs * (7 + cols)].copy_(self._pstage_host[:bs * (7 + cols)])
+            forward(bs)                          # warm-up: sizes every buffer before anything is captured
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, self.graph_pool):
+                self._pgraph_out[bs] = forward(bs)
+            if self.graph_pool is None:
+                self.graph_pool = graph.pool()
+            torch.cuda.synchronize()
+            self.graphs[bs] = graph
+            reset_context()
+        self.max_graph_bs = max_bs
+
+    def _run_decode_portions_graph(self, plan):
+        """A step in which every request brings exactly one token, through the captured graph of its padded size."""
+        B, bs, cols = len(plan), self.block_size, self._pstage_cols
+        padded = next(x for x in self.graph_bs if x >= B)
+        torch.cuda.current_stream().synchronize()            # the previous step's copy out of the pinned buffer is done
+        h = self._pstage_views(padded, self._pstage_host)
+        ids, pos, slots, past, states, tables = (h[k].numpy() for k in ("ids", "pos", "slots", "past", "states", "tables"))
+        ids[B:], pos[B:], slots[B:], past[B:] = 0, 0, -1, 0
+        states[B:] = self.num_state_slots
+        tables[:] = 0
+        for i, (seq, _) in enumerate(plan):
+            p = seq.num_computed_tokens
+            ids[i], pos[i], past[i], states[i] = seq.token_ids[p], p, p, seq.state_slot
+            table = seq.block_table
+            slots[i] = table[p // bs] * bs + p % bs
+            tables[i, :len(table)] = table
+        n = padded * (7 + cols)
+        self._pstage_dev[:n].copy_(self._pstage_host[:n], non_blocking=True)
+        self.graphs[padded].replay()
+        return self._pgraph_out[padded][:B]
 
     @torch.inference_mode()
     def run_portions(self, plan, want=None, sample: bool = True):
@@ -550,6 +626,12 @@ class ModelRunner:
         is drawn there -> one token id or None per pair.  want = per pair a list of positions inside its piece:
         -> fp32 logits [wanted, vocab] in that order (None when nothing is wanted); nothing is sampled."""
         bs = self.block_size
+        if (want is None and sample and self.graphs and len(plan) <= self.max_graph_bs
+                and all(count == 1 and seq.num_computed_tokens + 1 == seq.num_tokens
+                        and len(seq.block_table) <= self._pstage_cols for seq, count in plan)):
+            logits = self._run_decode_portions_graph(plan)
+            temperatures = self._to_device(torch.tensor([seq.temperature for seq, _ in plan], dtype=torch.float32))
+            return self.sampler(logits, temperatures).tolist()
         ids, pos, slots, seq_of, cu, past, state_slots = [], [], [], [], [0], [], []
         for i, (seq, count) in enumerate(plan):
             a, b = seq.num_computed_tokens, seq.num_computed_tokens + count
@@ -802,6 +884,7 @@ class ModelRunner:
         self.graph_vars = g
 
     portioned = False
+    graphs = None
     max_graph_bs = 0
     graph_has_head = False
     run_ahead = False

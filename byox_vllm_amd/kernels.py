@@ -457,6 +457,18 @@ def linear(x, w, bias=None, out=None, out_dtype=None, *, rows=None, a_rows=None,
     if n is None:
         n = w.size(-2) // (2 if epilogue == EPI_GLU else 1)
     M = x.size(0) if rows is None else rows
+    # prefill-sized plain products of a 16-bit model go where the engine sends its other many-row products: the vendor
+    # library, here with the result left in fp32
+    if (epilogue in (EPI_NONE, EPI_GLU) and batch == 1 and group_offsets is None and a_rows is None and bias is None and out is None
+            and rows is None and x.dtype == torch.bfloat16 and (out_dtype or x.dtype) in (torch.float32, torch.bfloat16)
+            and w.dim() == 2 and w.is_contiguous() and x.stride(0) % 8 == 0 and use_many_rows_path(M, K, n) and K % 8 == 0
+            and n % 8 == 0 and x.data_ptr() % 16 == 0):
+        if epilogue == EPI_GLU:      # [gate | up] rows from the library, activation and product in one pass over them
+            y = _linear_many_rows(x, w, M, 2 * n, K, torch.float32)
+            out = torch.empty(M, n, dtype=out_dtype or x.dtype, device=x.device)
+            check(lib().nv_act_mul_f32(ptr(y), ptr(out), M, n, act, _code32(out.dtype), stream()), "nv_act_mul_f32")
+            return out
+        return _linear_many_rows(x, w, M, n, K, out_dtype or x.dtype)
     grid_rows = M if group_offsets is None else (max_group_rows if max_group_rows is not None else M)
     out_dtype = out_dtype or x.dtype
     if out is None:
@@ -477,6 +489,18 @@ def linear(x, w, bias=None, out=None, out_dtype=None, *, rows=None, a_rows=None,
                           _code32(out_dtype), grid_rows, n, K, batch, a_batch_stride, w_batch_stride, out_batch_stride,
                           n if bias is not None and batch > 1 else 0, ptr(group_offsets), epilogue, act, ptr(gate),
                           gate_stride, cap, _code32(x.dtype), stream()), "nv_linear")
+    return out
+
+
+def _linear_many_rows(x, w, M, N, K, out_dtype):
+    ws = workspace(LT_WORKSPACE_BYTES, x.device, "gemm_lt")
+    out = torch.empty(M, N, dtype=out_dtype, device=x.device)
+    if out_dtype == torch.float32:
+        check(lib().nv_gemm_lt_f32out(ptr(x), x.stride(0), ptr(w), ptr(out), N, M, N, K, dtype_code(x.dtype), ptr(ws),
+                                      LT_WORKSPACE_BYTES, stream()), "nv_gemm_lt_f32out")
+    else:
+        check(lib().nv_gemm_lt(ptr(x), x.stride(0), ptr(w), None, ptr(out), N, M, N, K, dtype_code(x.dtype), ptr(ws),
+                               LT_WORKSPACE_BYTES, stream()), "nv_gemm_lt")
     return out
 
 

@@ -104,7 +104,7 @@ class RurutarLayer(nn.Module):
 class RurutarForCausalLM(nn.Module):
     portioned = True          # steps through ModelRunner.run_portions: prompt pieces and decoded tokens in one batch
     prefix_cache = False      # a recurrent state cannot be rebuilt from cached pages
-    kernel_sources = ("linear", "rowops", "gla", "latent_attn", "moe", "misc")     # csrc files this model launches
+    kernel_sources = ("linear", "rowops", "gla", "latent_attn", "moe", "misc", "gemm_lt")     # csrc files this model launches
 
     @staticmethod
     def config_from_json(raw: dict, path: str | None):

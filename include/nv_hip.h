@@ -326,6 +326,10 @@ int nv_allreduce_add_rmsnorm(nv_comm_t* comm, const void* x, const float* partia
                              const void* residual, const void* weight, void* out, void* residual_out, int64_t rows,
                              int hidden, float eps, int dtype, nv_stream_t stream);
 
+/* nv_gemm_lt with the result left in fp32 (no bias): for consumers that compute in fp32. */
+int nv_gemm_lt_f32out(const void* x, int64_t x_row_stride, const void* w_rowmajor, float* out, int64_t out_row_stride,
+                      int M, int N, int K, int dtype, void* workspace, size_t workspace_bytes, nv_stream_t stream);
+
 /* ---- kernels of models that keep the residual stream in fp32 and run in bf16 or true fp32 (dtype NV_BF16 / NV_F32) ----
  *
  * nv_linear: out[b][m][n] = epilogue(sum_k A[b][row(m)][k] * W[b][n][k] + bias[b][n]), fp32 accumulation.  Any M, N, K.
@@ -356,6 +360,9 @@ int nv_dyt_norm(float* x, const float* delta, int64_t delta_row_stride, const in
 /* RMS norm of fp32 rows: out = x / sqrt(mean(x^2) + eps) * w, rounded to the storage type. */
 int nv_rmsnorm_f32(const float* x, int64_t x_row_stride, const void* w, void* out, int64_t out_row_stride, int64_t rows,
                    int n, float eps, int dtype, nv_stream_t stream);
+
+/* out[m][j] = act(y[m][j]) * y[m][n + j] over fp32 rows [gate | up] of a plain product; act 0 SiLU, 1 tanh-form GELU. */
+int nv_act_mul_f32(const float* y, void* out, int64_t rows, int n, int act, int dtype, nv_stream_t stream);
 
 /* Sampler over fp32 logits: temperature 0 -> argmax (lowest index on ties), else Gumbel-max with noise hashed from
  * (seed, row, column). */

@@ -477,3 +477,25 @@ def test_fp32_sampler_argmax_and_temperature():
     draws = kernels.sample_f32(rows.to(DEV), torch.full((4000,), 0.5, device=DEV), seed=5).cpu()
     freq = torch.bincount(draws, minlength=3).double() / 4000
     assert torch.allclose(freq, torch.softmax(torch.tensor([4.0, 2.0, 0.0]).double(), 0), atol=0.03)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_captured_decode_steps_equal_eager_ones(dtype):
+    """Decode steps replayed from hipGraphs (padded batches, the spare state slot, one staging copy) give the tokens of
+    the eager engine, step after step, with prompt portions running eagerly between the replays."""
+    from byox_vllm_amd import LLM, SamplingParams
+    cfg = mixed_config()
+    weights = O.random_checkpoint(cfg, seed=21, decay_rank=8)
+    torch.manual_seed(5)
+    prompts = [torch.randint(0, cfg["vocab"], (n,)).tolist() for n in (37, 3, 18, 25, 9)]
+    params = [SamplingParams(temperature=0.0, max_tokens=n, ignore_eos=True) for n in (30, 41, 12, 25, 33)]
+    outs = []
+    for eager in (True, False):
+        conf = engine_config(cfg, weights, dtype, blocks=24, slots=4)
+        llm = LLM("synthetic", hf_config=conf.hf_config, state_dict=weights, kvcache_block_size=16, num_kvcache_blocks=24,
+                  max_num_seqs=4, num_state_slots=4, enforce_eager=eager, max_num_batched_tokens=32, max_model_len=128)
+        assert bool(llm.model_runner.graphs) == (not eager)
+        outs.append([o["token_ids"] for o in llm.generate(prompts, params, use_tqdm=False)])
+        llm._exit()
+    assert outs[0] == outs[1]
+    assert [len(t) for t in outs[0]] == [30, 41, 12, 25, 33]
