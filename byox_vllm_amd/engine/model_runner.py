@@ -580,6 +580,7 @@ class ModelRunner:
             return self.model.compute_logits(state, ramp[:bs], out_dtype=torch.float32)
 
         for bs in reversed(self.graph_bs):
+            self._pstage_host.zero_()            # the layout differs per size: no word of the previous one may stay
             h = views(bs, self._pstage_host)
             h["slots"].fill_(-1)
             h["states"].fill_(self.num_state_slots)
