@@ -181,15 +181,16 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(AttnArgs p) {
 // 16 threads per row, and every wavefront accumulates its share of the output columns.  Scores, maxima, sums and the
 // rescaling are fp32.  Queries and softmax weights enter the MFMAs as the sum of two bf16 numbers (value = hi + lo,
 // two MFMAs), so neither is rounded to 8 bits of mantissa; the cached rows are bf16 as stored.
-constexpr int ATT_KEYS = 64, ATT_PST = 72, ATT_SST = 68;
+// KEYS rows per tile: 64, or 32 where 64 would not fit the LDS beside wide latents (then two wavefronts compute scores)
 
 struct MfmaAttnArgs {
   AttnArgs a;
   int B, HQ, TQ, Dkp;
 };
 
-template <int NTILE>
+template <int NTILE, int KEYS>
 __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(MfmaAttnArgs q) {
+  constexpr int ATT_KEYS = KEYS, ATT_PST = KEYS + 8, ATT_SST = KEYS + 4, KPT = KEYS / 16;
   extern __shared__ u32x4 lds_raw[];
   const AttnArgs& p = q.a;
   const int Dk = p.rank + p.rot_dim, R = p.rank, Dq = q.Dkp + 8;
@@ -283,7 +284,7 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(MfmaAttnArgs q) {
     }
     __syncthreads();
     // S = Q K^T for this wavefront's 16 keys
-    {
+    if (16 * wv < ATT_KEYS) {
       f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
       const bf16_t* krow = sK + (16 * wv + c) * Dq + 8 * g;
       const bf16_t* qhi = sQhi + c * Dq + 8 * g;
@@ -297,14 +298,14 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(MfmaAttnArgs q) {
       for (int r = 0; r < 4; ++r) sS[(4 * g + r) * ATT_SST + 16 * wv + c] = acc[r] * p.scale;
     }
     __syncthreads();
-    // softmax statistics: 16 threads per row, 4 keys each
+    // softmax statistics: 16 threads per row, KEYS / 16 keys each
     {
-      float sv[4], m = -INFINITY;
+      float sv[KPT], m = -INFINITY;
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const int kp = j0 + 4 * skq + e;
+      for (int e = 0; e < KPT; ++e) {
+        const int kp = j0 + KPT * skq + e;
         const bool ok = s_valid && kp >= s_lo && kp <= s_pos;
-        sv[e] = ok ? sS[srow * ATT_SST + 4 * skq + e] : -INFINITY;
+        sv[e] = ok ? sS[srow * ATT_SST + KPT * skq + e] : -INFINITY;
         m = fmaxf(m, sv[e]);
       }
 #pragma unroll
@@ -313,12 +314,12 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(MfmaAttnArgs q) {
       const float m_new = fmaxf(m_old, m);
       float sum = 0.0f;
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
+      for (int e = 0; e < KPT; ++e) {
         const float pe = (sv[e] == -INFINITY) ? 0.0f : expf(sv[e] - m_new);
         sum += pe;
         const bf16_t hi = (bf16_t)pe;
-        sPhi[srow * ATT_PST + 4 * skq + e] = hi;
-        sPlo[srow * ATT_PST + 4 * skq + e] = (bf16_t)(pe - (float)hi);
+        sPhi[srow * ATT_PST + KPT * skq + e] = hi;
+        sPlo[srow * ATT_PST + KPT * skq + e] = (bf16_t)(pe - (float)hi);
       }
 #pragma unroll
       for (int o = 8; o > 0; o >>= 1) sum += __shfl_xor(sum, o, 64);
@@ -363,16 +364,16 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(MfmaAttnArgs q) {
   }
 }
 
-template <int NTILE>
+template <int NTILE, int KEYS>
 hipError_t launch_mfma_attn(const MfmaAttnArgs& q, dim3 grid, size_t lds, hipStream_t s) {
   static size_t allowed = 64 * 1024;
   if (lds > allowed) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&latent_attn_mfma_kernel<NTILE>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&latent_attn_mfma_kernel<NTILE, KEYS>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return e;
     allowed = lds;
   }
-  latent_attn_mfma_kernel<NTILE><<<grid, dim3(256), lds, s>>>(q);
+  latent_attn_mfma_kernel<NTILE, KEYS><<<grid, dim3(256), lds, s>>>(q);
   return hipSuccess;
 }
 
@@ -427,16 +428,23 @@ extern "C" int nv_latent_attn(const float* qa, const void* cache, const int32_t*
                     block_size, window, 0, 0, scale},
                    num_seqs, HQ, 16 / HQ, ((Dk + 31) / 32) * 32};
     const int Dq = q.Dkp + 8;
-    const size_t lds = (size_t)(2 * 16 * Dq + ATT_KEYS * Dq + rank * ATT_PST + 2 * 16 * ATT_PST) * 2 +
-                       (size_t)(16 * ATT_SST + 48) * 4;
+    auto lds_for = [&](int keys) {
+      return (size_t)(2 * 16 * Dq + keys * Dq + rank * (keys + 8) + 2 * 16 * (keys + 8)) * 2 + (size_t)(16 * (keys + 4) + 48) * 4;
+    };
+    const int keys = lds_for(64) <= 150 * 1024 ? 64 : 32;
+    const size_t lds = lds_for(keys);
     if (lds <= 150 * 1024) {
       const int64_t tiles = tokens / q.TQ + num_seqs;        // at most: every request may end in a partial tile
       NV_CHECK_ARG(tiles <= 65535, "nv_latent_attn: %lld tiles exceed one launch", (long long)tiles);
       dim3 grid((unsigned)((heads + HQ - 1) / HQ), (unsigned)tiles);
       const int ntile = (rank / 16 + 3) / 4;
-      hipError_t e = ntile <= 2   ? launch_mfma_attn<2>(q, grid, lds, (hipStream_t)stream)
-                     : ntile <= 4 ? launch_mfma_attn<4>(q, grid, lds, (hipStream_t)stream)
-                                  : launch_mfma_attn<8>(q, grid, lds, (hipStream_t)stream);
+      hipStream_t st = (hipStream_t)stream;
+      hipError_t e;
+      if (keys == 64)
+        e = ntile <= 2 ? launch_mfma_attn<2, 64>(q, grid, lds, st) : ntile <= 4 ? launch_mfma_attn<4, 64>(q, grid, lds, st)
+                                                                                 : launch_mfma_attn<8, 64>(q, grid, lds, st);
+      else
+        e = launch_mfma_attn<8, 32>(q, grid, lds, st);
       if (e != hipSuccess) {
         nv_set_error("nv_latent_attn: %s", hipGetErrorString(e));
         return NV_ERR_LAUNCH;

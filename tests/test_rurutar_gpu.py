@@ -231,7 +231,7 @@ def _paged(rows, block, num_blocks, seed):
 @pytest.mark.parametrize("H,R,r,window,block", [(3, 40, 8, 9, 16), (1, 20, 6, 5, 16), (5, 12, 2, 0, 32), (2, 200, 16, 70, 64),
                                                 # ranks that are multiples of 16: the matrix-core kernel in bf16
                                                 (6, 64, 8, 33, 16), (16, 32, 8, 5, 16), (2, 256, 32, 0, 32),
-                                                (20, 48, 16, 64, 64), (1, 16, 0, 3, 16)])
+                                                (20, 48, 16, 64, 64), (1, 16, 0, 3, 16), (4, 512, 32, 40, 64)])
 def test_latent_attention_prompt_pieces_and_single_tokens(dtype, H, R, r, window, block):
     from byox_vllm_amd import kernels
     torch.manual_seed(H * 10 + R)
