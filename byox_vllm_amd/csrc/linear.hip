@@ -103,17 +103,38 @@ __global__ __launch_bounds__(256) void linear_kernel(LinArgs p) {
 #pragma unroll
   for (int i = 0; i < 4; ++i) acc[i] = accu[i] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  for (int k0 = 0; k0 < p.K; k0 += KS) {
-    const int k = k0 + PER * g;
-    const F wf = load_frag<T>(wrow, k, p.K, p.vec_w);
-    F uf;
-    if constexpr (EPI == EPI_GLU) uf = load_frag<T>(urow, k, p.K, p.vec_w);
+  if (nsub == 1) {
+    // Few rows (decode): the loop would be one dependent weight load per k-step.  UNR k-steps per round: all fragments
+    // of a round are requested before the first MFMA waits for one, so the memory latency is paid once per round.
+    constexpr int UNR = 4;
+    for (int k0 = 0; k0 < p.K; k0 += KS * UNR) {
+      F wf[UNR], uf[UNR], xf[UNR];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      if (i < nsub) {
-        const F xf = load_frag<T>(arow[i], k, p.K, p.vec_a);
-        acc[i] = mma(wf, xf, acc[i]);
-        if constexpr (EPI == EPI_GLU) accu[i] = mma(uf, xf, accu[i]);
+      for (int u = 0; u < UNR; ++u) {
+        const int k = k0 + u * KS + PER * g;
+        wf[u] = load_frag<T>(wrow, k, p.K, p.vec_w);
+        if constexpr (EPI == EPI_GLU) uf[u] = load_frag<T>(urow, k, p.K, p.vec_w);
+        xf[u] = load_frag<T>(arow[0], k, p.K, p.vec_a);
+      }
+#pragma unroll
+      for (int u = 0; u < UNR; ++u) {
+        acc[0] = mma(wf[u], xf[u], acc[0]);
+        if constexpr (EPI == EPI_GLU) accu[0] = mma(uf[u], xf[u], accu[0]);
+      }
+    }
+  } else {
+    for (int k0 = 0; k0 < p.K; k0 += KS) {
+      const int k = k0 + PER * g;
+      const F wf = load_frag<T>(wrow, k, p.K, p.vec_w);
+      F uf;
+      if constexpr (EPI == EPI_GLU) uf = load_frag<T>(urow, k, p.K, p.vec_w);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        if (i < nsub) {
+          const F xf = load_frag<T>(arow[i], k, p.K, p.vec_a);
+          acc[i] = mma(wf, xf, acc[i]);
+          if constexpr (EPI == EPI_GLU) accu[i] = mma(uf, xf, accu[i]);
+        }
       }
     }
   }
