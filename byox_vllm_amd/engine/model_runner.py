@@ -533,6 +533,9 @@ class ModelRunner:
             free, total = torch.cuda.mem_get_info()
             room = int(total * config.gpu_memory_utilization - (total - free)) - state_bytes
             config.num_kvcache_blocks = max(1, room // max(block_bytes, 1)) if pages else 1
+            # more than every request at full length cannot be used
+            config.num_kvcache_blocks = min(config.num_kvcache_blocks,
+                                            config.max_num_seqs * (-(-config.max_model_len // self.block_size) + 1))
         assert config.num_kvcache_blocks > 0
         rows = config.num_kvcache_blocks * self.block_size
         for m in pages:

@@ -499,3 +499,56 @@ def test_captured_decode_steps_equal_eager_ones(dtype):
         llm._exit()
     assert outs[0] == outs[1]
     assert [len(t) for t in outs[0]] == [30, 41, 12, 25, 33]
+
+
+def test_command_line_generation_and_trace_replay_from_a_model_folder(tmp_path):
+    """A model folder (config.json + model.safetensors in bf16) through the two command-line entry points, each in a
+    process of its own: `python -m byox_vllm_amd generate` against the oracle's greedy continuation, bin/trace_run
+    against the oracle's logits for a replayed schedule with pieces, a pause and a request that ends early."""
+    import json
+    import os
+    import subprocess
+    import sys
+
+    import numpy as np
+    from safetensors.torch import save_file
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    cfg = aligned_config()
+    weights = O.random_checkpoint(cfg, seed=31, decay_rank=16)
+    model = tmp_path / "model"
+    model.mkdir()
+    with open(model / "config.json", "w") as f:
+        json.dump(cfg, f)
+    save_file({k: v.contiguous() for k, v in weights.items()}, str(model / "model.safetensors"))
+    torch.manual_seed(3)
+    a = torch.randint(0, cfg["vocab"], (70,)).tolist()
+    b = torch.randint(0, cfg["vocab"], (9,)).tolist()
+
+    run = subprocess.run([sys.executable, "-m", "byox_vllm_amd", "generate", "--model", str(model), "--dtype", "float32",
+                          "--prompt-ids", ",".join(map(str, b)), "--max-tokens", "6", "--block-size", "16", "--eager"],
+                         cwd=root, capture_output=True, text=True, timeout=600)
+    assert run.returncode == 0, run.stderr[-3000:]
+    line = json.loads([ln for ln in run.stdout.splitlines() if ln.startswith("{")][0])
+    tokens = list(b)
+    for tok in line["token_ids"]:
+        logits = O.forward(tokens, weights, cfg)[-1]
+        assert logits.max().item() - logits[tok].item() <= 1e-3
+        tokens.append(tok)
+    assert len(line["token_ids"]) == 6
+
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": a[:40], "want": [0, 39]}], "end": []},
+             {"step": 1, "entries": [{"id": "b", "tokens": b[:2], "want": []}, {"id": "a", "tokens": a[40:41], "want": [0]}], "end": []},
+             {"step": 2, "entries": [{"id": "b", "tokens": b[2:], "want": [6]}], "end": ["b"]},
+             {"step": 3, "entries": [{"id": "a", "tokens": a[41:], "want": [0, 28]}, {"id": "c", "tokens": b, "want": [8]}], "end": ["a", "c"]}]
+    for dtype, tol in (("float32", F32_TOL), ("bfloat16", BF16_TOL)):
+        out = tmp_path / ("out_" + dtype)
+        run = subprocess.run([os.path.join(root, "bin", "trace_run"), "--model", str(model), "--dtype", dtype, "--out", str(out),
+                              "--max-tokens", "192"], input="\n".join(json.dumps(s) for s in steps) + "\n", cwd=root,
+                             capture_output=True, text=True, timeout=600)
+        assert run.returncode == 0, run.stderr[-3000:]
+        assert [ln for ln in run.stdout.splitlines() if ln.startswith("done")] == [f"done {i}" for i in range(4)]
+        wa, wb = O.forward(a, weights, cfg).float(), O.forward(b, weights, cfg).float()
+        expect = {0: wa[[0, 39]], 1: wa[[40]], 2: wb[[8]], 3: torch.cat([wa[[41, 69]], wb[[8]]])}
+        for i, want in expect.items():
+            got = torch.from_numpy(np.fromfile(out / f"{i}.f32", dtype="<f4").reshape(-1, cfg["vocab"]))
+            assert got.shape == want.shape and row_error(got, want) < tol, (dtype, i)
