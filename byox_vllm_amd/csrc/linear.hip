@@ -8,6 +8,8 @@
 // layout: lane (c, g) holds row c, k = k0 + 8 g .. + 8), so there is no LDS stage; the 4 wavefronts re-read the A rows
 // through the L1.  D[n][m] is accumulated (the weight fragment is the first operand), which leaves every lane with
 // four consecutive output columns.
+#include <stdlib.h>
+
 #include "anyt.h"
 
 namespace {
@@ -164,6 +166,150 @@ __global__ __launch_bounds__(256) void linear_kernel(LinArgs p) {
   }
 }
 
+
+// Many rows (prefill, expert groups): a 128 x 128 output tile per workgroup, operands staged through LDS in K-blocks of
+// 32 (two buffers: the next block is fetched into registers while the current one is multiplied), wavefront (wm, wn)
+// owns 64 x 64 of the tile.  With the gated epilogue the weight tile holds 64 gate rows and their 64 up rows, and a
+// wavefront owns 64 x 32 of gate and of up.  bf16 operands whose rows split into 16-byte pieces only.
+constexpr int TBM = 128, TBK = 32, TST = 40;    // LDS row stride in elements (80 bytes: 16-byte aligned, spreads banks)
+
+template <typename TO, int EPI>
+__global__ __launch_bounds__(256) void linear_tile_kernel(LinArgs p) {
+  constexpr bool GLU = EPI == EPI_GLU;
+  constexpr int NOUT = GLU ? 64 : 128;          // output columns per workgroup
+  constexpr int NJ = GLU ? 2 : 4;               // 16-column sub-tiles per wavefront
+  __shared__ __attribute__((aligned(16))) bf16_t sA[2][TBM * TST];
+  __shared__ __attribute__((aligned(16))) bf16_t sW[2][TBM * TST];
+  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  const int c = lane & 15, g = lane >> 4, wm = wv >> 1, wn = wv & 1;
+  const int z = blockIdx.z;
+  int64_t lo = 0, hi = p.M;
+  if (p.group_off) {
+    lo = p.group_off[z];
+    hi = p.group_off[z + 1];
+  }
+  const int64_t mbase = lo + (int64_t)blockIdx.y * TBM;
+  if (mbase >= hi) return;
+  const int n0 = blockIdx.x * NOUT;
+  const bf16_t* A = reinterpret_cast<const bf16_t*>(p.a) + z * p.a_bs;
+  const bf16_t* W = reinterpret_cast<const bf16_t*>(p.w) + z * p.w_bs;
+  // this thread's two 16-byte pieces of each operand tile: rows r0 and r0 + 64, K offset 8 * ch
+  const int r0 = tid >> 2, ch = tid & 3;
+  const bf16_t* ap[2];
+  const bf16_t* wp[2];
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int r = r0 + 64 * h;
+    const int64_t s = mbase + r;
+    ap[h] = s < hi ? A + (int64_t)(p.a_rows ? p.a_rows[s] : s) * p.a_rs + 8 * ch : nullptr;
+    int wrow;                                    // weight row behind tile row r
+    if constexpr (GLU) wrow = r < 64 ? n0 + r : p.N + n0 + (r - 64);
+    else wrow = n0 + r;
+    const bool in = GLU ? (n0 + (r & 63) < p.N) : (wrow < p.N);
+    wp[h] = in ? W + (int64_t)wrow * p.w_rs + 8 * ch : nullptr;
+  }
+  auto fetch = [&](const bf16_t* q, int k0) -> u32x4 {
+    if (q == nullptr || k0 + 8 * ch + 8 > p.K) {
+      u32x4 v = u32x4{0u, 0u, 0u, 0u};
+      if (q != nullptr && k0 + 8 * ch < p.K) {      // a K that is no multiple of 32 ends inside this piece
+        uint16_t* e = reinterpret_cast<uint16_t*>(&v);
+        for (int i = 0; i < 8 && k0 + 8 * ch + i < p.K; ++i) e[i] = reinterpret_cast<const uint16_t*>(q + k0)[i];
+      }
+      return v;
+    }
+    return *reinterpret_cast<const u32x4*>(q + k0);
+  };
+  f32x4 acc[4][NJ], accu[4][NJ];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) acc[i][j] = accu[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  u32x4 ra[2], rw[2];
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    ra[h] = fetch(ap[h], 0);
+    rw[h] = fetch(wp[h], 0);
+  }
+  int buf = 0;
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    *reinterpret_cast<u32x4*>(&sA[0][(r0 + 64 * h) * TST + 8 * ch]) = ra[h];
+    *reinterpret_cast<u32x4*>(&sW[0][(r0 + 64 * h) * TST + 8 * ch]) = rw[h];
+  }
+  __syncthreads();
+  for (int k0 = 0; k0 < p.K; k0 += TBK) {
+    const bool more = k0 + TBK < p.K;
+    if (more) {
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        ra[h] = fetch(ap[h], k0 + TBK);
+        rw[h] = fetch(wp[h], k0 + TBK);
+      }
+    }
+    bf16x8 af[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) af[i] = *reinterpret_cast<const bf16x8*>(&sA[buf][(64 * wm + 16 * i + c) * TST + 8 * g]);
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+      const int wr = GLU ? 32 * wn + 16 * j : 64 * wn + 16 * j;
+      const bf16x8 wf = *reinterpret_cast<const bf16x8*>(&sW[buf][(wr + c) * TST + 8 * g]);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[i][j] = mma(wf, af[i], acc[i][j]);
+      if constexpr (GLU) {
+        const bf16x8 uf = *reinterpret_cast<const bf16x8*>(&sW[buf][(64 + wr + c) * TST + 8 * g]);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) accu[i][j] = mma(uf, af[i], accu[i][j]);
+      }
+    }
+    if (more) {
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        *reinterpret_cast<u32x4*>(&sA[buf ^ 1][(r0 + 64 * h) * TST + 8 * ch]) = ra[h];
+        *reinterpret_cast<u32x4*>(&sW[buf ^ 1][(r0 + 64 * h) * TST + 8 * ch]) = rw[h];
+      }
+    }
+    __syncthreads();
+    buf ^= 1;
+  }
+
+  TO* O = reinterpret_cast<TO*>(p.out) + z * p.out_bs;
+  const bf16_t* bias = p.bias ? reinterpret_cast<const bf16_t*>(p.bias) + z * p.bias_bs : nullptr;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int64_t s = mbase + 64 * wm + 16 * i + c;
+    if (s >= hi) continue;
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int n = n0 + (GLU ? 32 * wn : 64 * wn) + 16 * j + 4 * g + r;
+        if (n >= p.N) continue;
+        float v = acc[i][j][r];
+        if (bias) v += ld_f32<bf16_t>(bias + n);
+        if constexpr (GLU) {
+          v = (p.act == 1 ? gelu_tanh_f32(v) : silu_f32(v)) * accu[i][j][r];
+        } else if constexpr (EPI == EPI_SOFTCAP) {
+          v = p.epi_c * tanhf(v / p.epi_c);
+        } else if constexpr (EPI == EPI_ROW_GATE) {
+          v *= sigmoid_f32(p.epi_ptr[s * p.epi_rs + z]);
+        }
+        st_f32<TO>(O + s * p.out_rs + n, v);
+      }
+    }
+  }
+}
+
+template <typename TO>
+int launch_tile(const LinArgs& p, int epi, int batch, hipStream_t s) {
+  const unsigned my = (unsigned)((p.M + TBM - 1) / TBM);
+  if (epi == EPI_GLU) linear_tile_kernel<TO, EPI_GLU><<<dim3((p.N + 63) / 64, my, batch), dim3(256), 0, s>>>(p);
+  else if (epi == EPI_NONE) linear_tile_kernel<TO, EPI_NONE><<<dim3((p.N + 127) / 128, my, batch), dim3(256), 0, s>>>(p);
+  else if (epi == EPI_SOFTCAP) linear_tile_kernel<TO, EPI_SOFTCAP><<<dim3((p.N + 127) / 128, my, batch), dim3(256), 0, s>>>(p);
+  else linear_tile_kernel<TO, EPI_ROW_GATE><<<dim3((p.N + 127) / 128, my, batch), dim3(256), 0, s>>>(p);
+  return 0;
+}
+
 template <typename T, typename TO>
 int launch_epi(const LinArgs& p, int epi, dim3 grid, hipStream_t s) {
   switch (epi) {
@@ -202,6 +348,13 @@ extern "C" int nv_linear(const void* a, int64_t a_row_stride, const int32_t* a_r
   p.vec_w = (uintptr_t)w % 16 == 0 && w_row_stride % per == 0 && (w_batch_stride * esz) % 16 == 0;
   dim3 grid((unsigned)((N + 63) / 64), (unsigned)mtiles, (unsigned)batch);
   hipStream_t s = (hipStream_t)stream;
+  // many rows of 16-byte-aligned bf16: the LDS-tiled kernel (a group's rows are not known here: M bounds them)
+  if (dtype == NV_BF16 && M >= 256 && p.vec_a && p.vec_w && K % 8 == 0 && getenv("NV_LINEAR_TILE_OFF") == nullptr) {
+    if (out_dtype == NV_BF16) launch_tile<bf16_t>(p, epilogue, batch, s);
+    else launch_tile<float>(p, epilogue, batch, s);
+    NV_CHECK_LAUNCH();
+    return NV_OK;
+  }
   if (dtype == NV_BF16) {
     if (out_dtype == NV_BF16) launch_epi<bf16_t, bf16_t>(p, epilogue, grid, s);
     else launch_epi<bf16_t, float>(p, epilogue, grid, s);

@@ -552,3 +552,49 @@ def test_command_line_generation_and_trace_replay_from_a_model_folder(tmp_path):
         for i, want in expect.items():
             got = torch.from_numpy(np.fromfile(out / f"{i}.f32", dtype="<f4").reshape(-1, cfg["vocab"]))
             assert got.shape == want.shape and row_error(got, want) < tol, (dtype, i)
+
+
+@pytest.mark.parametrize("M,N,K", [(256, 128, 32), (300, 200, 72), (1000, 72, 256), (513, 130, 40)])
+def test_linear_many_rows_go_through_the_tiled_kernel(M, N, K):
+    """From 256 rows of 16-byte-aligned bf16 on, nv_linear stages its operands through LDS: plain, gated, soft-capped,
+    with bias, with row and column tails and a K that is no multiple of the K-block."""
+    from byox_vllm_amd import kernels
+    torch.manual_seed(M + N)
+    x, w, b = (torch.randn(M, K) / 4).bfloat16(), torch.randn(2 * N, K).bfloat16(), torch.randn(N).bfloat16()
+    xd, wd = x.to(DEV), w.to(DEV)
+    want = x.double() @ w[:N].double().T + b.double()
+    got = kernels.linear(xd, wd[:N], b.to(DEV), out_dtype=torch.float32).cpu()
+    assert torch.allclose(got.double(), want, rtol=1e-5, atol=1e-4)
+    g, u = x.double() @ w[:N].double().T, x.double() @ w[N:].double().T
+    got = kernels.linear(xd, wd, epilogue=kernels.EPI_GLU, act=kernels.ACT_GELU_TANH, out_dtype=torch.float32).cpu()
+    assert torch.allclose(got.double(), O.gelu_tanh(g) * u, rtol=1e-4, atol=1e-4)
+    got = kernels.linear(xd, wd[:N], epilogue=kernels.EPI_SOFTCAP, cap=2.0).cpu()
+    assert torch.allclose(got.double(), 2.0 * torch.tanh(g / 2.0), rtol=2e-2, atol=2e-2)
+
+
+def test_linear_many_rows_groups_batches_and_gates():
+    from byox_vllm_amd import kernels
+    torch.manual_seed(12)
+    T, K, N, sizes = 400, 48, 40, [0, 700, 3, 129, 260]
+    E, total = len(sizes), sum(sizes)
+    x, w = (torch.randn(T, K) / 4).bfloat16(), torch.randn(E, 2 * N, K).bfloat16()
+    rows = torch.randint(0, T, (total,), dtype=torch.int32)
+    offsets = torch.tensor([0] + torch.tensor(sizes).cumsum(0).tolist(), dtype=torch.int32)
+    got = kernels.linear(x.to(DEV), w.to(DEV), out_dtype=torch.float32, rows=total, a_rows=rows.to(DEV), batch=E,
+                         w_batch_stride=2 * N * K, group_offsets=offsets.to(DEV), max_group_rows=max(sizes),
+                         epilogue=kernels.EPI_GLU).cpu()
+    for e in range(E):
+        lo, hi = offsets[e], offsets[e + 1]
+        xe = x.double()[rows[lo:hi].long()]
+        want = O.silu(xe @ w[e, :N].double().T) * (xe @ w[e, N:].double().T)
+        assert torch.allclose(got[lo:hi].double(), want, rtol=1e-4, atol=1e-4), e
+    H, Kh, Nh = 3, 24, 20
+    xh, wh, gate = (torch.randn(T, H * Kh) / 4).bfloat16(), torch.randn(H, Nh, Kh).bfloat16(), torch.randn(T, H)
+    want = torch.stack([xh.double().view(T, H, Kh)[:, h] @ wh[h].double().T for h in range(H)], 1)
+    want = want * torch.sigmoid(gate.double()[:, :, None])
+    out = torch.zeros(T, H * Nh, dtype=torch.float32, device=DEV)
+    gd = gate.to(DEV)
+    kernels.linear(xh.to(DEV), wh.to(DEV), out=out, out_dtype=torch.float32, batch=H, a_batch_stride=Kh,
+                   w_batch_stride=Nh * Kh, out_batch_stride=Nh, n=Nh, epilogue=kernels.EPI_ROW_GATE, gate=gd,
+                   gate_stride=gd.stride(0))
+    assert torch.allclose(out.cpu().double().view(T, H, Nh), want, rtol=1e-4, atol=1e-4)
