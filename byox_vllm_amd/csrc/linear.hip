@@ -310,6 +310,91 @@ int launch_tile(const LinArgs& p, int epi, int batch, hipStream_t s) {
   return 0;
 }
 
+
+// Up to 16 rows per (group of) product: the launch is bound by how many weight loads are in flight, so the four
+// wavefronts of a workgroup share ONE 16-column tile and split K between them (four times the workgroups of the
+// general kernel, a quarter of the dependent rounds each); the partial sums meet in LDS and wavefront 0 finishes.
+template <typename T, typename TO, int EPI>
+__global__ __launch_bounds__(256) void linear_fewrow_kernel(LinArgs p) {
+  typedef typename Frag<T>::type F;
+  constexpr int KS = Frag<T>::KS, PER = Frag<T>::PER, UNR = 4;
+  constexpr bool GLU = EPI == EPI_GLU;
+  __shared__ float part[2][4][256];
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int c = lane & 15, g = lane >> 4;
+  const int z = blockIdx.z;
+  int64_t lo = 0, hi = p.M;
+  if (p.group_off) {
+    lo = p.group_off[z];
+    hi = p.group_off[z + 1];
+  }
+  if (lo >= hi) return;
+  const int n0 = blockIdx.x * 16;
+  const T* A = reinterpret_cast<const T*>(p.a) + z * p.a_bs;
+  const T* W = reinterpret_cast<const T*>(p.w) + z * p.w_bs;
+  const T* wrow = (n0 + c < p.N) ? W + (int64_t)(n0 + c) * p.w_rs : nullptr;
+  const T* urow = nullptr;
+  if constexpr (GLU) urow = (n0 + c < p.N) ? W + (int64_t)(p.N + n0 + c) * p.w_rs : nullptr;
+  const int64_t s = lo + c;
+  const T* arow = s < hi ? A + (int64_t)(p.a_rows ? p.a_rows[s] : s) * p.a_rs : nullptr;
+  // this wavefront's share of K, in whole rounds
+  const int round = KS * UNR;
+  const int rounds = (p.K + round - 1) / round;
+  const int k_lo = ((rounds * wv) / 4) * round, k_hi = min(p.K, ((rounds * (wv + 1)) / 4) * round);
+  f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f}, accu = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int k0 = k_lo; k0 < k_hi; k0 += round) {
+    F wf[UNR], uf[UNR], xf[UNR];
+#pragma unroll
+    for (int u = 0; u < UNR; ++u) {
+      const int k = k0 + u * KS + PER * g;
+      wf[u] = load_frag<T>(wrow, k, k_hi, p.vec_w);
+      if constexpr (GLU) uf[u] = load_frag<T>(urow, k, k_hi, p.vec_w);
+      xf[u] = load_frag<T>(arow, k, k_hi, p.vec_a);
+    }
+#pragma unroll
+    for (int u = 0; u < UNR; ++u) {
+      acc = mma(wf[u], xf[u], acc);
+      if constexpr (GLU) accu = mma(uf[u], xf[u], accu);
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    part[0][wv][4 * lane + r] = acc[r];
+    if constexpr (GLU) part[1][wv][4 * lane + r] = accu[r];
+  }
+  __syncthreads();
+  if (wv != 0 || s >= hi) return;
+  TO* O = reinterpret_cast<TO*>(p.out) + z * p.out_bs;
+  const T* bias = p.bias ? reinterpret_cast<const T*>(p.bias) + z * p.bias_bs : nullptr;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int n = n0 + 4 * g + r;
+    if (n >= p.N) continue;
+    float v = part[0][0][4 * lane + r] + part[0][1][4 * lane + r] + part[0][2][4 * lane + r] + part[0][3][4 * lane + r];
+    if (bias) v += ld_f32<T>(bias + n);
+    if constexpr (GLU) {
+      const float u = part[1][0][4 * lane + r] + part[1][1][4 * lane + r] + part[1][2][4 * lane + r] + part[1][3][4 * lane + r];
+      v = (p.act == 1 ? gelu_tanh_f32(v) : silu_f32(v)) * u;
+    } else if constexpr (EPI == EPI_SOFTCAP) {
+      v = p.epi_c * tanhf(v / p.epi_c);
+    } else if constexpr (EPI == EPI_ROW_GATE) {
+      v *= sigmoid_f32(p.epi_ptr[s * p.epi_rs + z]);
+    }
+    st_f32<TO>(O + s * p.out_rs + n, v);
+  }
+}
+
+template <typename T, typename TO>
+int launch_fewrow(const LinArgs& p, int epi, dim3 grid, hipStream_t s) {
+  switch (epi) {
+    case EPI_NONE: linear_fewrow_kernel<T, TO, EPI_NONE><<<grid, dim3(256), 0, s>>>(p); break;
+    case EPI_GLU: linear_fewrow_kernel<T, TO, EPI_GLU><<<grid, dim3(256), 0, s>>>(p); break;
+    case EPI_SOFTCAP: linear_fewrow_kernel<T, TO, EPI_SOFTCAP><<<grid, dim3(256), 0, s>>>(p); break;
+    default: linear_fewrow_kernel<T, TO, EPI_ROW_GATE><<<grid, dim3(256), 0, s>>>(p); break;
+  }
+  return 0;
+}
+
 template <typename T, typename TO>
 int launch_epi(const LinArgs& p, int epi, dim3 grid, hipStream_t s) {
   switch (epi) {
@@ -352,6 +437,19 @@ extern "C" int nv_linear(const void* a, int64_t a_row_stride, const int32_t* a_r
   if (dtype == NV_BF16 && M >= 256 && p.vec_a && p.vec_w && K % 8 == 0 && getenv("NV_LINEAR_TILE_OFF") == nullptr) {
     if (out_dtype == NV_BF16) launch_tile<bf16_t>(p, epilogue, batch, s);
     else launch_tile<float>(p, epilogue, batch, s);
+    NV_CHECK_LAUNCH();
+    return NV_OK;
+  }
+  // at most 16 rows per product and a K worth splitting: one 16-column tile per workgroup, K split over its wavefronts
+  if (M <= 16 && K >= 256 && (N + 15) / 16 <= 1048576) {
+    dim3 g16((unsigned)((N + 15) / 16), 1, (unsigned)batch);
+    if (dtype == NV_BF16) {
+      if (out_dtype == NV_BF16) launch_fewrow<bf16_t, bf16_t>(p, epilogue, g16, s);
+      else launch_fewrow<bf16_t, float>(p, epilogue, g16, s);
+    } else {
+      if (out_dtype == NV_BF16) launch_fewrow<float, bf16_t>(p, epilogue, g16, s);
+      else launch_fewrow<float, float>(p, epilogue, g16, s);
+    }
     NV_CHECK_LAUNCH();
     return NV_OK;
   }

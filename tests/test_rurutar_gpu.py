@@ -598,3 +598,28 @@ def test_linear_many_rows_groups_batches_and_gates():
                    w_batch_stride=Nh * Kh, out_batch_stride=Nh, n=Nh, epilogue=kernels.EPI_ROW_GATE, gate=gd,
                    gate_stride=gd.stride(0))
     assert torch.allclose(out.cpu().double().view(T, H, Nh), want, rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("M,N,K", [(1, 40, 256), (8, 130, 1000), (16, 64, 2048), (5, 7, 300)])
+def test_linear_few_rows_split_k_over_the_wavefronts(dtype, M, N, K):
+    """Up to 16 rows and K >= 256: one 16-column tile per workgroup with K split over its wavefronts; plain, gated,
+    grouped over gathered rows, with the per-head gate."""
+    from byox_vllm_amd import kernels
+    torch.manual_seed(M * 7 + N)
+    x, w, b = (torch.randn(M, K) / 8).to(dtype), torch.randn(2 * N, K).to(dtype), torch.randn(N).to(dtype)
+    xd, wd = x.to(DEV), w.to(DEV)
+    g, u = x.double() @ w[:N].double().T, x.double() @ w[N:].double().T
+    got = kernels.linear(xd, wd[:N], b.to(DEV), out_dtype=torch.float32).cpu()
+    assert torch.allclose(got.double(), g + b.double(), rtol=1e-4, atol=1e-4)
+    got = kernels.linear(xd, wd, epilogue=kernels.EPI_GLU, out_dtype=torch.float32).cpu()
+    assert torch.allclose(got.double(), O.silu(g) * u, rtol=1e-4, atol=1e-4)
+    E, sizes = 3, [M, 0, max(1, M // 2)]
+    we = torch.randn(E, N, K).to(dtype)
+    rows = torch.randint(0, M, (sum(sizes),), dtype=torch.int32)
+    offsets = torch.tensor([0, sizes[0], sizes[0], sum(sizes)], dtype=torch.int32)
+    got = kernels.linear(xd, we.to(DEV), out_dtype=torch.float32, rows=sum(sizes), a_rows=rows.to(DEV), batch=E,
+                         w_batch_stride=N * K, group_offsets=offsets.to(DEV), max_group_rows=M).cpu()
+    for e in range(E):
+        lo, hi = offsets[e], offsets[e + 1]
+        assert torch.allclose(got[lo:hi].double(), x.double()[rows[lo:hi].long()] @ we[e].double().T, rtol=1e-4, atol=1e-4)
