@@ -59,6 +59,8 @@ def main(argv=None) -> int:
         step = json.loads(line)
         plan, want = [], []
         for entry in step["entries"]:
+            if not entry["tokens"]:
+                continue                      # nothing to run for this request in this step
             seq = live.get(entry["id"])
             if seq is None:
                 seq = live[entry["id"]] = Sequence(entry["tokens"], BLOCK)
