@@ -288,6 +288,7 @@ def run_generate_workload(args):
 ARCH_COMPARE_SIZES = {
     "w1024": (1024, 8, 8, 2048, 64),
     "w2048": (2048, 8, 8, 2048, 64),
+    "w1024-b64": (1024, 8, 64, 256, 64),       # a decode batch of 64 short requests
 }
 
 

@@ -311,15 +311,16 @@ int launch_tile(const LinArgs& p, int epi, int batch, hipStream_t s) {
 }
 
 
-// Up to 16 rows per (group of) product: the launch is bound by how many weight loads are in flight, so the four
+// Up to 64 rows per (group of) product: the launch is bound by how many weight loads are in flight, so the four
 // wavefronts of a workgroup share ONE 16-column tile and split K between them (four times the workgroups of the
 // general kernel, a quarter of the dependent rounds each); the partial sums meet in LDS and wavefront 0 finishes.
-template <typename T, typename TO, int EPI>
+// NSUB = 16-row sub-tiles (1: at most 16 rows, 4: at most 64).
+template <typename T, typename TO, int EPI, int NSUB>
 __global__ __launch_bounds__(256) void linear_fewrow_kernel(LinArgs p) {
   typedef typename Frag<T>::type F;
   constexpr int KS = Frag<T>::KS, PER = Frag<T>::PER, UNR = 4;
   constexpr bool GLU = EPI == EPI_GLU;
-  __shared__ float part[2][4][256];
+  __shared__ float part[GLU ? 2 : 1][4][NSUB][256];
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const int c = lane & 15, g = lane >> 4;
   const int z = blockIdx.z;
@@ -329,70 +330,104 @@ __global__ __launch_bounds__(256) void linear_fewrow_kernel(LinArgs p) {
     hi = p.group_off[z + 1];
   }
   if (lo >= hi) return;
+  const int nsub = (int)((hi - lo + 15) / 16 < NSUB ? (hi - lo + 15) / 16 : NSUB);
   const int n0 = blockIdx.x * 16;
   const T* A = reinterpret_cast<const T*>(p.a) + z * p.a_bs;
   const T* W = reinterpret_cast<const T*>(p.w) + z * p.w_bs;
   const T* wrow = (n0 + c < p.N) ? W + (int64_t)(n0 + c) * p.w_rs : nullptr;
   const T* urow = nullptr;
   if constexpr (GLU) urow = (n0 + c < p.N) ? W + (int64_t)(p.N + n0 + c) * p.w_rs : nullptr;
-  const int64_t s = lo + c;
-  const T* arow = s < hi ? A + (int64_t)(p.a_rows ? p.a_rows[s] : s) * p.a_rs : nullptr;
+  const T* arow[NSUB];
+#pragma unroll
+  for (int i = 0; i < NSUB; ++i) {
+    const int64_t s = lo + 16 * i + c;
+    arow[i] = s < hi ? A + (int64_t)(p.a_rows ? p.a_rows[s] : s) * p.a_rs : nullptr;
+  }
   // this wavefront's share of K, in whole rounds
   const int round = KS * UNR;
   const int rounds = (p.K + round - 1) / round;
   const int k_lo = ((rounds * wv) / 4) * round, k_hi = min(p.K, ((rounds * (wv + 1)) / 4) * round);
-  f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f}, accu = f32x4{0.f, 0.f, 0.f, 0.f};
+  f32x4 acc[NSUB], accu[NSUB];
+#pragma unroll
+  for (int i = 0; i < NSUB; ++i) acc[i] = accu[i] = f32x4{0.f, 0.f, 0.f, 0.f};
   for (int k0 = k_lo; k0 < k_hi; k0 += round) {
-    F wf[UNR], uf[UNR], xf[UNR];
+    F wf[UNR], uf[UNR], xf[NSUB][UNR];
 #pragma unroll
     for (int u = 0; u < UNR; ++u) {
       const int k = k0 + u * KS + PER * g;
       wf[u] = load_frag<T>(wrow, k, k_hi, p.vec_w);
       if constexpr (GLU) uf[u] = load_frag<T>(urow, k, k_hi, p.vec_w);
-      xf[u] = load_frag<T>(arow, k, k_hi, p.vec_a);
+#pragma unroll
+      for (int i = 0; i < NSUB; ++i)
+        if (i < nsub) xf[i][u] = load_frag<T>(arow[i], k, k_hi, p.vec_a);
     }
 #pragma unroll
     for (int u = 0; u < UNR; ++u) {
-      acc = mma(wf[u], xf[u], acc);
-      if constexpr (GLU) accu = mma(uf[u], xf[u], accu);
+#pragma unroll
+      for (int i = 0; i < NSUB; ++i) {
+        if (i < nsub) {
+          acc[i] = mma(wf[u], xf[i][u], acc[i]);
+          if constexpr (GLU) accu[i] = mma(uf[u], xf[i][u], accu[i]);
+        }
+      }
     }
   }
 #pragma unroll
-  for (int r = 0; r < 4; ++r) {
-    part[0][wv][4 * lane + r] = acc[r];
-    if constexpr (GLU) part[1][wv][4 * lane + r] = accu[r];
+  for (int i = 0; i < NSUB; ++i) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      part[0][wv][i][4 * lane + r] = acc[i][r];
+      if constexpr (GLU) part[1][wv][i][4 * lane + r] = accu[i][r];
+    }
   }
   __syncthreads();
-  if (wv != 0 || s >= hi) return;
+  if (wv != 0) return;
   TO* O = reinterpret_cast<TO*>(p.out) + z * p.out_bs;
   const T* bias = p.bias ? reinterpret_cast<const T*>(p.bias) + z * p.bias_bs : nullptr;
 #pragma unroll
-  for (int r = 0; r < 4; ++r) {
-    const int n = n0 + 4 * g + r;
-    if (n >= p.N) continue;
-    float v = part[0][0][4 * lane + r] + part[0][1][4 * lane + r] + part[0][2][4 * lane + r] + part[0][3][4 * lane + r];
-    if (bias) v += ld_f32<T>(bias + n);
-    if constexpr (GLU) {
-      const float u = part[1][0][4 * lane + r] + part[1][1][4 * lane + r] + part[1][2][4 * lane + r] + part[1][3][4 * lane + r];
-      v = (p.act == 1 ? gelu_tanh_f32(v) : silu_f32(v)) * u;
-    } else if constexpr (EPI == EPI_SOFTCAP) {
-      v = p.epi_c * tanhf(v / p.epi_c);
-    } else if constexpr (EPI == EPI_ROW_GATE) {
-      v *= sigmoid_f32(p.epi_ptr[s * p.epi_rs + z]);
+  for (int i = 0; i < NSUB; ++i) {
+    const int64_t s = lo + 16 * i + c;
+    if (i >= nsub || s >= hi) continue;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int n = n0 + 4 * g + r;
+      if (n >= p.N) continue;
+      const int e = 4 * lane + r;
+      float v = part[0][0][i][e] + part[0][1][i][e] + part[0][2][i][e] + part[0][3][i][e];
+      if (bias) v += ld_f32<T>(bias + n);
+      if constexpr (GLU) {
+        const float u = part[1][0][i][e] + part[1][1][i][e] + part[1][2][i][e] + part[1][3][i][e];
+        v = (p.act == 1 ? gelu_tanh_f32(v) : silu_f32(v)) * u;
+      } else if constexpr (EPI == EPI_SOFTCAP) {
+        v = p.epi_c * tanhf(v / p.epi_c);
+      } else if constexpr (EPI == EPI_ROW_GATE) {
+        v *= sigmoid_f32(p.epi_ptr[s * p.epi_rs + z]);
+      }
+      st_f32<TO>(O + s * p.out_rs + n, v);
     }
-    st_f32<TO>(O + s * p.out_rs + n, v);
   }
 }
 
-template <typename T, typename TO>
+template <typename T, typename TO, int NSUB>
 int launch_fewrow(const LinArgs& p, int epi, dim3 grid, hipStream_t s) {
   switch (epi) {
-    case EPI_NONE: linear_fewrow_kernel<T, TO, EPI_NONE><<<grid, dim3(256), 0, s>>>(p); break;
-    case EPI_GLU: linear_fewrow_kernel<T, TO, EPI_GLU><<<grid, dim3(256), 0, s>>>(p); break;
-    case EPI_SOFTCAP: linear_fewrow_kernel<T, TO, EPI_SOFTCAP><<<grid, dim3(256), 0, s>>>(p); break;
-    default: linear_fewrow_kernel<T, TO, EPI_ROW_GATE><<<grid, dim3(256), 0, s>>>(p); break;
+    case EPI_NONE: linear_fewrow_kernel<T, TO, EPI_NONE, NSUB><<<grid, dim3(256), 0, s>>>(p); break;
+    case EPI_GLU: linear_fewrow_kernel<T, TO, EPI_GLU, NSUB><<<grid, dim3(256), 0, s>>>(p); break;
+    case EPI_SOFTCAP: linear_fewrow_kernel<T, TO, EPI_SOFTCAP, NSUB><<<grid, dim3(256), 0, s>>>(p); break;
+    default: linear_fewrow_kernel<T, TO, EPI_ROW_GATE, NSUB><<<grid, dim3(256), 0, s>>>(p); break;
   }
   return 0;
+}
+
+template <int NSUB>
+void launch_fewrow_any(const LinArgs& p, int epi, dim3 grid, int dtype, int out_dtype, hipStream_t s) {
+  if (dtype == NV_BF16) {
+    if (out_dtype == NV_BF16) launch_fewrow<bf16_t, bf16_t, NSUB>(p, epi, grid, s);
+    else launch_fewrow<bf16_t, float, NSUB>(p, epi, grid, s);
+  } else {
+    if (out_dtype == NV_BF16) launch_fewrow<float, bf16_t, NSUB>(p, epi, grid, s);
+    else launch_fewrow<float, float, NSUB>(p, epi, grid, s);
+  }
 }
 
 template <typename T, typename TO>
@@ -433,23 +468,18 @@ extern "C" int nv_linear(const void* a, int64_t a_row_stride, const int32_t* a_r
   p.vec_w = (uintptr_t)w % 16 == 0 && w_row_stride % per == 0 && (w_batch_stride * esz) % 16 == 0;
   dim3 grid((unsigned)((N + 63) / 64), (unsigned)mtiles, (unsigned)batch);
   hipStream_t s = (hipStream_t)stream;
-  // many rows of 16-byte-aligned bf16: the LDS-tiled kernel (a group's rows are not known here: M bounds them)
-  if (dtype == NV_BF16 && M >= 256 && p.vec_a && p.vec_w && K % 8 == 0 && getenv("NV_LINEAR_TILE_OFF") == nullptr) {
+  // more than 64 rows of 16-byte-aligned bf16: the LDS-tiled kernel (a group's rows are not known here: M bounds them)
+  if (dtype == NV_BF16 && M > 64 && p.vec_a && p.vec_w && K % 8 == 0 && getenv("NV_LINEAR_TILE_OFF") == nullptr) {
     if (out_dtype == NV_BF16) launch_tile<bf16_t>(p, epilogue, batch, s);
     else launch_tile<float>(p, epilogue, batch, s);
     NV_CHECK_LAUNCH();
     return NV_OK;
   }
-  // at most 16 rows per product and a K worth splitting: one 16-column tile per workgroup, K split over its wavefronts
-  if (M <= 16 && K >= 256 && (N + 15) / 16 <= 1048576) {
+  // at most 64 rows per product and a K worth splitting: one 16-column tile per workgroup, K split over its wavefronts
+  if (M <= 64 && K >= 256 && (N + 15) / 16 <= 1048576) {
     dim3 g16((unsigned)((N + 15) / 16), 1, (unsigned)batch);
-    if (dtype == NV_BF16) {
-      if (out_dtype == NV_BF16) launch_fewrow<bf16_t, bf16_t>(p, epilogue, g16, s);
-      else launch_fewrow<bf16_t, float>(p, epilogue, g16, s);
-    } else {
-      if (out_dtype == NV_BF16) launch_fewrow<float, bf16_t>(p, epilogue, g16, s);
-      else launch_fewrow<float, float>(p, epilogue, g16, s);
-    }
+    if (M <= 16) launch_fewrow_any<1>(p, epilogue, g16, dtype, out_dtype, s);
+    else launch_fewrow_any<4>(p, epilogue, g16, dtype, out_dtype, s);
     NV_CHECK_LAUNCH();
     return NV_OK;
   }

@@ -554,9 +554,9 @@ def test_command_line_generation_and_trace_replay_from_a_model_folder(tmp_path):
             assert got.shape == want.shape and row_error(got, want) < tol, (dtype, i)
 
 
-@pytest.mark.parametrize("M,N,K", [(256, 128, 32), (300, 200, 72), (1000, 72, 256), (513, 130, 40)])
+@pytest.mark.parametrize("M,N,K", [(256, 128, 32), (300, 200, 72), (1000, 72, 256), (513, 130, 40), (65, 40, 64), (130, 16, 512)])
 def test_linear_many_rows_go_through_the_tiled_kernel(M, N, K):
-    """From 256 rows of 16-byte-aligned bf16 on, nv_linear stages its operands through LDS: plain, gated, soft-capped,
+    """From 65 rows of 16-byte-aligned bf16 on, nv_linear stages its operands through LDS: plain, gated, soft-capped,
     with bias, with row and column tails and a K that is no multiple of the K-block."""
     from byox_vllm_amd import kernels
     torch.manual_seed(M + N)
@@ -601,10 +601,11 @@ def test_linear_many_rows_groups_batches_and_gates():
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("M,N,K", [(1, 40, 256), (8, 130, 1000), (16, 64, 2048), (5, 7, 300)])
+@pytest.mark.parametrize("M,N,K", [(1, 40, 256), (8, 130, 1000), (16, 64, 2048), (5, 7, 300), (17, 40, 512), (64, 72, 260),
+                                   (33, 130, 1024)])
 def test_linear_few_rows_split_k_over_the_wavefronts(dtype, M, N, K):
-    """Up to 16 rows and K >= 256: one 16-column tile per workgroup with K split over its wavefronts; plain, gated,
-    grouped over gathered rows, with the per-head gate."""
+    """Up to 64 rows and K >= 256: one 16-column tile per workgroup with K split over its wavefronts; plain, gated,
+    grouped over gathered rows."""
     from byox_vllm_amd import kernels
     torch.manual_seed(M * 7 + N)
     x, w, b = (torch.randn(M, K) / 8).to(dtype), torch.randn(2 * N, K).to(dtype), torch.randn(N).to(dtype)
