@@ -176,6 +176,9 @@ class Scheduler:
             admitted += 1
             budget -= count
             free -= bm.blocks_short(seq, count)
+        if not plan and (self.running or self.waiting):
+            raise RuntimeError("no request can take a step: the block pool or the state slots are too small for the "
+                               "oldest request alone (num_kvcache_blocks, num_state_slots)")
         return self.commit(plan)
 
     def advance(self, plan: list[tuple[Sequence, int]], token_ids: list[int | None]) -> list[Sequence]:

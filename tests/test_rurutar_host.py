@@ -283,3 +283,15 @@ def test_engine_config_helper_marks_the_model_portioned():
     cfg = odd_config()
     c = engine_config(cfg, O.random_checkpoint(cfg, seed=4, decay_rank=5), torch.bfloat16)
     assert c.portioned and c.hf_config.layers[0]["mixer"]["decay_rank"] == 5 and os.path.basename(c.model) == "synthetic"
+
+
+def test_own_policy_says_so_when_the_pool_cannot_hold_one_request():
+    s = _scheduler(blocks=2, slots=1, budget=64)
+    a = Sequence(list(range(40)), 16)
+    a.max_tokens, a.ignore_eos = 4, True
+    s.add(a)
+    plan = s.schedule_portions()
+    assert [(q.seq_id, n) for q, n in plan] == [(a.seq_id, 32)]      # what two pages hold
+    s.advance(plan, [None])
+    with pytest.raises(RuntimeError):
+        s.schedule_portions()                                         # the third page does not exist
