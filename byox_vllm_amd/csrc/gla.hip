@@ -98,29 +98,35 @@ __global__ __launch_bounds__(1024) void gla_kernel(GlaArgs p) {
 // channels per read; the RMS norm's sum over vdim is taken for the sixteen tokens at once (three barriers per chunk).
 constexpr int GLA_TC = 16;
 
-constexpr int gla_col_threads(int dmax) { return dmax >= 64 ? 256 : 512; }   // bounded by registers per thread
+constexpr int gla_col_threads(int per_thread) { return per_thread >= 64 ? 256 : 512; }   // by state registers per thread
 
-template <typename T, int DMAX>
-__global__ __launch_bounds__(gla_col_threads(DMAX)) void gla_col_kernel(GlaArgs p) {
+template <typename T, int DMAX, int CS>
+__global__ __launch_bounds__(gla_col_threads(DMAX / CS)) void gla_col_kernel(GlaArgs p) {
+  // CS: the key channels of a column are split over CS threads (more wavefronts per (request, head), shorter per-token
+  // chains); their partial o_t meet in LDS once per chunk of tokens.  vdp = threads per split, whole wavefronts.
+  constexpr int DC = DMAX / CS;
   extern __shared__ float4 lds4[];
   float* lds = reinterpret_cast<float*>(lds4);
   const int vd = p.vdim;
+  const int tid = threadIdx.x, nthr = blockDim.x, vdp = nthr / CS;
   float* sa = lds;                       // [TC][DMAX]
   float* sk = sa + GLA_TC * DMAX;
   float* sq = sk + GLA_TC * DMAX;
-  float* sred = sq + GLA_TC * DMAX;      // [TC][waves]
+  float* sred = sq + GLA_TC * DMAX;      // [TC][waves of one split]
+  float* so = sred + GLA_TC * (vdp >> 6);   // [CS][TC][vdp] partial outputs (CS > 1)
   const int h = blockIdx.x, b = blockIdx.y;
-  const int tid = threadIdx.x, nthr = blockDim.x, wv = tid >> 6, nw = nthr >> 6;
-  const bool active = tid < vd;
-  const int col = active ? tid : 0;
+  const int v = tid % vdp, cs = tid / vdp, wv = v >> 6, nw = vdp >> 6;
+  const int cb = cs * DC;
+  const bool active = v < vd;
+  const int col = active ? v : 0;
   const int t0 = p.cu_q[b], t1 = p.cu_q[b + 1];
   if (t1 <= t0) return;
   float* S_g = p.state + ((int64_t)p.slots[b] * p.H + h) * p.dim * vd;
-  float S[DMAX];
+  float S[DC];
   const bool fresh = p.past[b] == 0;
 #pragma unroll
-  for (int i = 0; i < DMAX; ++i) S[i] = (active && i < p.dim && !fresh) ? S_g[(int64_t)i * vd + tid] : 0.0f;
-  const float nw_v = active ? ld_f32<T>(reinterpret_cast<const T*>(p.norm_w) + tid) : 0.0f;
+  for (int i = 0; i < DC; ++i) S[i] = (active && cb + i < p.dim && !fresh) ? S_g[(int64_t)(cb + i) * vd + v] : 0.0f;
+  const float nw_v = active ? ld_f32<T>(reinterpret_cast<const T*>(p.norm_w) + v) : 0.0f;
   for (int c0 = t0; c0 < t1; c0 += GLA_TC) {
     const int nt = min(GLA_TC, t1 - c0);
     // this thread's own v and gate values of the chunk: sixteen loads in flight, no LDS
@@ -131,20 +137,19 @@ __global__ __launch_bounds__(gla_col_threads(DMAX)) void gla_col_kernel(GlaArgs 
       if (j < nt) {
         const float* row = p.proj + (int64_t)(c0 + j) * p.proj_rs;
         vreg[j] = row[p.v_off + h * vd + col];
-        greg[j] = row[p.g_off + h * vd + col];
+        if (cs == 0) greg[j] = row[p.g_off + h * vd + col];
       }
     }
     __syncthreads();                     // the previous chunk's rows are no longer read
-    // decay, k and q rows of the chunk, four elements per thread and round so that the loads overlap
+    // decay, k and q rows of the chunk, four elements per thread and step so that the loads overlap
     for (int base = tid * 4; base < nt * DMAX; base += nthr * 4) {
       const int j = base / DMAX, i = base % DMAX;          // DMAX is a multiple of 4: the four share a token
       float z4[4], k4[4], q4[4];
-      const bool live = j < nt;
-      const float* row = p.proj + (int64_t)(c0 + (live ? j : 0)) * p.proj_rs;
-      const float* zr = p.z + (int64_t)(c0 + (live ? j : 0)) * p.z_rs;
+      const float* row = p.proj + (int64_t)(c0 + j) * p.proj_rs;
+      const float* zr = p.z + (int64_t)(c0 + j) * p.z_rs;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        const bool in = live && i + e < p.dim;
+        const bool in = i + e < p.dim;
         const int ch = h * p.dim + (in ? i + e : 0);
         z4[e] = zr[ch];
         k4[e] = in ? row[p.k_off + ch] : 0.0f;
@@ -162,11 +167,11 @@ __global__ __launch_bounds__(gla_col_threads(DMAX)) void gla_col_kernel(GlaArgs 
       float acc0 = 0.0f, acc1 = 0.0f;
       if (j < nt) {
         const float vv = vreg[j];
-        const float4* a4 = reinterpret_cast<const float4*>(sa + j * DMAX);
-        const float4* k4 = reinterpret_cast<const float4*>(sk + j * DMAX);
-        const float4* q4 = reinterpret_cast<const float4*>(sq + j * DMAX);
+        const float4* a4 = reinterpret_cast<const float4*>(sa + j * DMAX + cb);
+        const float4* k4 = reinterpret_cast<const float4*>(sk + j * DMAX + cb);
+        const float4* q4 = reinterpret_cast<const float4*>(sq + j * DMAX + cb);
 #pragma unroll
-        for (int i = 0; i < DMAX / 4; ++i) {
+        for (int i = 0; i < DC / 4; ++i) {
           const float4 a = a4[i], k = k4[i], q = q4[i];
           S[4 * i + 0] = a.x * S[4 * i + 0] + k.x * vv;
           S[4 * i + 1] = a.y * S[4 * i + 1] + k.y * vv;
@@ -179,18 +184,34 @@ __global__ __launch_bounds__(gla_col_threads(DMAX)) void gla_col_kernel(GlaArgs 
         }
       }
       o[j] = acc0 + acc1;
-      const float ss = wave_sum(active ? o[j] * o[j] : 0.0f);
-      if ((tid & 63) == 0) sred[j * nw + wv] = ss;
+    }
+    if constexpr (CS > 1) {
+#pragma unroll
+      for (int j = 0; j < GLA_TC; ++j) so[(cs * GLA_TC + j) * vdp + v] = o[j];
+      __syncthreads();
+    }
+    if (cs == 0) {
+#pragma unroll
+      for (int j = 0; j < GLA_TC; ++j) {
+        if constexpr (CS > 1) {
+          float t = 0.0f;
+#pragma unroll
+          for (int q = 0; q < CS; ++q) t += so[(q * GLA_TC + j) * vdp + v];
+          o[j] = t;
+        }
+        const float ss = wave_sum(active ? o[j] * o[j] : 0.0f);
+        if ((tid & 63) == 0) sred[j * nw + wv] = ss;
+      }
     }
     __syncthreads();
-    if (active) {
+    if (cs == 0 && active) {
 #pragma unroll
       for (int j = 0; j < GLA_TC; ++j) {
         if (j < nt) {
           float ss = 0.0f;
           for (int w = 0; w < nw; ++w) ss += sred[j * nw + w];
           const float inv = 1.0f / sqrtf(ss / (float)vd + p.eps);
-          st_f32<T>(reinterpret_cast<T*>(p.out) + (int64_t)(c0 + j) * p.H * vd + h * vd + tid,
+          st_f32<T>(reinterpret_cast<T*>(p.out) + (int64_t)(c0 + j) * p.H * vd + h * vd + v,
                     o[j] * inv * nw_v * silu_f32(greg[j]));
         }
       }
@@ -198,20 +219,27 @@ __global__ __launch_bounds__(gla_col_threads(DMAX)) void gla_col_kernel(GlaArgs 
   }
   if (active) {
 #pragma unroll
-    for (int i = 0; i < DMAX; ++i)
-      if (i < p.dim) S_g[(int64_t)i * vd + tid] = S[i];
+    for (int i = 0; i < DC; ++i)
+      if (cb + i < p.dim) S_g[(int64_t)(cb + i) * vd + v] = S[i];
   }
 }
 
-template <typename T>
-int launch_col(const GlaArgs& p, int dmax, dim3 grid, int threads, size_t lds, hipStream_t s) {
-  switch (dmax) {
-    case 16: gla_col_kernel<T, 16><<<grid, dim3(threads), lds, s>>>(p); break;
-    case 32: gla_col_kernel<T, 32><<<grid, dim3(threads), lds, s>>>(p); break;
-    case 64: gla_col_kernel<T, 64><<<grid, dim3(threads), lds, s>>>(p); break;
-    default: gla_col_kernel<T, 128><<<grid, dim3(threads), lds, s>>>(p); break;
-  }
+template <typename T, int DMAX>
+int launch_col_cs(const GlaArgs& p, int cs, dim3 grid, int threads, size_t lds, hipStream_t s) {
+  if (cs == 4) gla_col_kernel<T, DMAX, 4><<<grid, dim3(threads), lds, s>>>(p);
+  else if (cs == 2) gla_col_kernel<T, DMAX, 2><<<grid, dim3(threads), lds, s>>>(p);
+  else gla_col_kernel<T, DMAX, 1><<<grid, dim3(threads), lds, s>>>(p);
   return 0;
+}
+
+template <typename T>
+int launch_col(const GlaArgs& p, int dmax, int cs, dim3 grid, int threads, size_t lds, hipStream_t s) {
+  switch (dmax) {
+    case 16: return launch_col_cs<T, 16>(p, cs, grid, threads, lds, s);
+    case 32: return launch_col_cs<T, 32>(p, cs, grid, threads, lds, s);
+    case 64: return launch_col_cs<T, 64>(p, cs, grid, threads, lds, s);
+    default: return launch_col_cs<T, 128>(p, cs, grid, threads, lds, s);
+  }
 }
 
 template <typename T>
@@ -238,15 +266,18 @@ extern "C" int nv_gla_recurrent(const float* proj, int64_t proj_row_stride, int 
                "nv_gla_recurrent: bad shape heads=%d dim=%d vdim=%d seqs=%d", heads, dim, vdim, num_seqs);
   NV_CHECK_ARG(tau > 0.0f, "nv_gla_recurrent: tau must be positive");
   if (num_seqs == 0) return NV_OK;
-  if (dim <= 128) {     // one state column per thread
+  if (dim <= 128) {     // one state column per thread (or per CS threads)
     int dmax = 16;
     while (dmax < dim) dmax *= 2;
-    const int threads = ((vdim + 63) / 64) * 64;
-    const size_t lds = (size_t)(GLA_TC * 3 * dmax + GLA_TC * (threads / 64)) * sizeof(float);
-    if (lds <= 64 * 1024 && threads <= gla_col_threads(dmax)) {
+    const int vdp = ((vdim + 63) / 64) * 64;
+    int cs = 1;
+    while (cs < 4 && vdp * cs * 2 <= 256 && dmax / (cs * 2) >= 16) cs *= 2;
+    const int threads = vdp * cs;
+    const size_t lds = (size_t)(GLA_TC * 3 * dmax + GLA_TC * (vdp / 64) + (cs > 1 ? cs * GLA_TC * vdp : 0)) * sizeof(float);
+    if (lds <= 64 * 1024 && threads <= gla_col_threads(dmax / cs)) {
       GlaArgs p{proj, proj_row_stride, q_off, k_off, v_off, g_off, z, z_row_stride, state, cu_q, past_lens, state_slots,
                 norm_w, out, heads, dim, vdim, 1, 1.0f / tau, q_scale, eps};
-      NV_DISPATCH_T(dtype, launch_col<T>(p, dmax, dim3(heads, num_seqs), threads, lds, (hipStream_t)stream));
+      NV_DISPATCH_T(dtype, launch_col<T>(p, dmax, cs, dim3(heads, num_seqs), threads, lds, (hipStream_t)stream));
       NV_CHECK_LAUNCH();
       return NV_OK;
     }
