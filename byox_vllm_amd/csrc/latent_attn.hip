@@ -201,7 +201,7 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(MfmaAttnArgs q) {
   bf16_t* sPhi = sVt + R * ATT_PST;
   bf16_t* sPlo = sPhi + 16 * ATT_PST;
   float* sS = reinterpret_cast<float*>(sPlo + 16 * ATT_PST);
-  float* sm = sS + 16 * ATT_SST;
+  float* sm = sS + 2 * 16 * ATT_SST;      // two score tiles: the second holds the other feature half (32-key tiles)
   float* sl = sm + 16;
   float* scorr = sl + 16;
   const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6, c = lane & 15, g = lane >> 4;
@@ -283,19 +283,25 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(MfmaAttnArgs q) {
       }
     }
     __syncthreads();
-    // S = Q K^T for this wavefront's 16 keys
-    if (16 * wv < ATT_KEYS) {
+    // S = Q K^T: with 64 keys wavefront w takes keys 16 w ..; with 32 keys the wavefront pairs (0, 1) and (2, 3) take
+    // the two halves of the feature dimension and their partial scores are summed in the softmax step
+    {
+      constexpr int KW = ATT_KEYS / 16;             // wavefronts one pass over the keys needs
+      constexpr int PARTS = 4 / KW;                 // feature ranges (1 or 2)
+      const int kw = wv % KW, part = wv / KW;
+      const int steps = q.Dkp / 32;
+      const int f_lo = (steps * part) / PARTS * 32, f_hi = (steps * (part + 1)) / PARTS * 32;
       f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
-      const bf16_t* krow = sK + (16 * wv + c) * Dq + 8 * g;
+      const bf16_t* krow = sK + (16 * kw + c) * Dq + 8 * g;
       const bf16_t* qhi = sQhi + c * Dq + 8 * g;
       const bf16_t* qlo = sQlo + c * Dq + 8 * g;
-      for (int ks = 0; ks < q.Dkp; ks += 32) {
+      for (int ks = f_lo; ks < f_hi; ks += 32) {
         const bf16x8 kf = *reinterpret_cast<const bf16x8*>(krow + ks);
         acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<const bf16x8*>(qhi + ks), kf, acc, 0, 0, 0);
         acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<const bf16x8*>(qlo + ks), kf, acc, 0, 0, 0);
       }
 #pragma unroll
-      for (int r = 0; r < 4; ++r) sS[(4 * g + r) * ATT_SST + 16 * wv + c] = acc[r] * p.scale;
+      for (int r = 0; r < 4; ++r) sS[part * 16 * ATT_SST + (4 * g + r) * ATT_SST + 16 * kw + c] = acc[r] * p.scale;
     }
     __syncthreads();
     // softmax statistics: 16 threads per row, KEYS / 16 keys each
@@ -305,7 +311,11 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(MfmaAttnArgs q) {
       for (int e = 0; e < KPT; ++e) {
         const int kp = j0 + KPT * skq + e;
         const bool ok = s_valid && kp >= s_lo && kp <= s_pos;
-        sv[e] = ok ? sS[srow * ATT_SST + KPT * skq + e] : -INFINITY;
+        sv[e] = -INFINITY;
+        if (ok) {
+          sv[e] = sS[srow * ATT_SST + KPT * skq + e];
+          if constexpr (ATT_KEYS == 32) sv[e] += sS[16 * ATT_SST + srow * ATT_SST + KPT * skq + e];
+        }
         m = fmaxf(m, sv[e]);
       }
 #pragma unroll
@@ -429,7 +439,7 @@ extern "C" int nv_latent_attn(const float* qa, const void* cache, const int32_t*
                    num_seqs, HQ, 16 / HQ, ((Dk + 31) / 32) * 32};
     const int Dq = q.Dkp + 8;
     auto lds_for = [&](int keys) {
-      return (size_t)(2 * 16 * Dq + keys * Dq + rank * (keys + 8) + 2 * 16 * (keys + 8)) * 2 + (size_t)(16 * (keys + 4) + 48) * 4;
+      return (size_t)(2 * 16 * Dq + keys * Dq + rank * (keys + 8) + 2 * 16 * (keys + 8)) * 2 + (size_t)(2 * 16 * (keys + 4) + 48) * 4;
     };
     const int keys = lds_for(64) <= 150 * 1024 ? 64 : 32;
     const size_t lds = lds_for(keys);
