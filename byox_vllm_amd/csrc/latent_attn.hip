@@ -252,37 +252,42 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(MfmaAttnArgs q) {
   const int chunks = Dk / 8;
   __syncthreads();
 
-  for (int j0 = kmin; j0 <= kmax; j0 += ATT_KEYS) {
-    // stage the key rows: consecutive threads take consecutive keys (conflict-free transposed stores); four loads are
-    // issued before the first is stored, so their latencies overlap
-    for (int i0 = tid; i0 < ATT_KEYS * chunks; i0 += 4 * 256) {
-      u32x4 v[4];
+  // Key rows travel memory -> registers -> LDS; the loads of the NEXT tile are issued before this tile is multiplied,
+  // so their latency hides behind the MFMAs.  Consecutive threads take consecutive keys (conflict-free transposed
+  // stores).  NCH bounds the 16-byte pieces per thread and tile (the launcher checks it).
+  constexpr int NCH = 10;
+  const int pieces = ATT_KEYS * chunks;
+  u32x4 stage[NCH];
+  auto fetch_tile = [&](int j0) {
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const int i = i0 + u * 256;
-        const int key = i % ATT_KEYS, f8 = i / ATT_KEYS;
-        const int kp = j0 + key;
-        v[u] = u32x4{0u, 0u, 0u, 0u};
-        if (f8 < chunks && kp <= kmax) {
-          const int64_t row = (int64_t)table[kp / p.block_size] * p.block_size + kp % p.block_size;
-          v[u] = *reinterpret_cast<const u32x4*>(cache + row * Dk + f8 * 8);
-        }
+    for (int u = 0; u < NCH; ++u) {
+      const int i = tid + u * 256;
+      const int key = i % ATT_KEYS, f8 = i / ATT_KEYS;
+      const int kp = j0 + key;
+      stage[u] = u32x4{0u, 0u, 0u, 0u};
+      if (i < pieces && kp <= kmax) {
+        const int64_t row = (int64_t)table[kp / p.block_size] * p.block_size + kp % p.block_size;
+        stage[u] = *reinterpret_cast<const u32x4*>(cache + row * Dk + f8 * 8);
       }
+    }
+  };
+  fetch_tile(kmin);
+  for (int j0 = kmin; j0 <= kmax; j0 += ATT_KEYS) {
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const int i = i0 + u * 256;
-        const int key = i % ATT_KEYS, f8 = i / ATT_KEYS;
-        if (f8 >= chunks) continue;
-        *reinterpret_cast<u32x4*>(sK + key * Dq + f8 * 8) = v[u];
-        if (f8 * 8 < R) {
-          const uint16_t* e16 = reinterpret_cast<const uint16_t*>(&v[u]);
-          uint16_t* dst = reinterpret_cast<uint16_t*>(sVt) + (f8 * 8) * ATT_PST + key;
+    for (int u = 0; u < NCH; ++u) {
+      const int i = tid + u * 256;
+      const int key = i % ATT_KEYS, f8 = i / ATT_KEYS;
+      if (i >= pieces) continue;
+      *reinterpret_cast<u32x4*>(sK + key * Dq + f8 * 8) = stage[u];
+      if (f8 * 8 < R) {
+        const uint16_t* e16 = reinterpret_cast<const uint16_t*>(&stage[u]);
+        uint16_t* dst = reinterpret_cast<uint16_t*>(sVt) + (f8 * 8) * ATT_PST + key;
 #pragma unroll
-          for (int e = 0; e < 8; ++e) dst[e * ATT_PST] = e16[e];
-        }
+        for (int e = 0; e < 8; ++e) dst[e * ATT_PST] = e16[e];
       }
     }
     __syncthreads();
+    if (j0 + ATT_KEYS <= kmax) fetch_tile(j0 + ATT_KEYS);
     // S = Q K^T: with 64 keys wavefront w takes keys 16 w ..; with 32 keys the wavefront pairs (0, 1) and (2, 3) take
     // the two halves of the feature dimension and their partial scores are summed in the softmax step
     {
@@ -443,7 +448,7 @@ extern "C" int nv_latent_attn(const float* qa, const void* cache, const int32_t*
     };
     const int keys = lds_for(64) <= 150 * 1024 ? 64 : 32;
     const size_t lds = lds_for(keys);
-    if (lds <= 150 * 1024) {
+    if (lds <= 150 * 1024 && keys * (Dk / 8) <= 10 * 256) {
       const int64_t tiles = tokens / q.TQ + num_seqs;        // at most: every request may end in a partial tile
       NV_CHECK_ARG(tiles <= 65535, "nv_latent_attn: %lld tiles exceed one launch", (long long)tiles);
       dim3 grid((unsigned)((heads + HQ - 1) / HQ), (unsigned)tiles);
