@@ -80,6 +80,15 @@ _PROTOS = {
     "nv_moe_route": (_i, [_p, _i64, _p, _p, _i64, _i, _i, _p]),
     "nv_moe_sort": (_i, [_p, _i64, _i, _i, _p, _p, _p, _p]),
     "nv_moe_combine": (_i, [_p, _p, _p, _i, _p, _p, _i64, _p, _i64, _i, _p]),
+    "nv_embed_sinusoid": (_i, [_p, _p, _p, _p, _p, _i64, _i, _i, _i64, _i, _p]),
+    "nv_hc_norm": (_i, [_p, _i, _i, _p, _i64, _p, _p, _p, _i, _f, _p, _p, _i64, _i, _i64, _i, _p]),
+    "nv_token_shift": (_i, [_p, _p, _p, _p, _p, _p, _p, _p, _i64, _i, _i, _p]),
+    "nv_group_rmsnorm_f32": (_i, [_p, _i64, _p, _p, _i64, _i64, _i, _i, _f, _i, _p]),
+    "nv_qk_norm_store": (_i, [_p, _i64, _i, _i, _i, _p, _p, _p, _f, _f, _p, _p, _p, _i64, _i, _i, _i, _i, _i, _p]),
+    "nv_window_attn": (_i, [_p, _p, _p, _i, _p, _p, _p, _p, _i64, _i64, _i, _i, _i, _i, _i, _i, _i, _f, _f, _i, _p]),
+    "nv_causal_conv": (_i, [_p, _i64, _p, _p, _p, _p, _p, _p, _p, _p, _i64, _p, _i64, _i64, _i, _i, _i, _i, _p]),
+    "nv_rglru_scan": (_i, [_p, _i64, _p, _i64, _p, _i64, _p, _p, _p, _p, _p, _p, _i64, _i, _i, _i, _f, _f, _i, _p]),
+    "nv_ssd_scan": (_i, [_p, _i64, _p, _i64, _p, _i64, _p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _p]),
 }
 
 _lib = None

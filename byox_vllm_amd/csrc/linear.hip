@@ -34,7 +34,18 @@ struct LinArgs {
   int vec_a, vec_w;
 };
 
-enum { EPI_NONE = 0, EPI_GLU = 1, EPI_SOFTCAP = 2, EPI_ROW_GATE = 3 };
+enum { EPI_NONE = 0, EPI_GLU = 1, EPI_SOFTCAP = 2, EPI_ROW_GATE = 3, EPI_ACT = 4 };
+
+// EPI_ACT: an element-wise function of the product.  act 0 SiLU, 1 tanh-form GELU, 2 xIELU with its two positive
+// coefficients at epi_ptr (a z^2 + z/2 above zero, b (exp(z) - 1 - z) + z/2 below), 3 multiplication by epi_c.
+__device__ __forceinline__ float unary_act(float v, int act, const float* prm, float c) {
+  switch (act) {
+    case 0: return silu_f32(v);
+    case 1: return gelu_tanh_f32(v);
+    case 2: return v > 0.0f ? prm[0] * v * v + 0.5f * v : prm[1] * (expm1f(v) - v) + 0.5f * v;
+    default: return v * c;
+  }
+}
 
 template <typename T> struct Frag;
 template <> struct Frag<bf16_t> {
@@ -160,6 +171,8 @@ __global__ __launch_bounds__(256) void linear_kernel(LinArgs p) {
         v = p.epi_c * tanhf(v / p.epi_c);
       } else if constexpr (EPI == EPI_ROW_GATE) {
         v *= sigmoid_f32(p.epi_ptr[s * p.epi_rs + z]);
+      } else if constexpr (EPI == EPI_ACT) {
+        v = unary_act(v, p.act, p.epi_ptr, p.epi_c);
       }
       st_f32<TO>(O + s * p.out_rs + n, v);
     }
@@ -293,6 +306,8 @@ __global__ __launch_bounds__(256) void linear_tile_kernel(LinArgs p) {
           v = p.epi_c * tanhf(v / p.epi_c);
         } else if constexpr (EPI == EPI_ROW_GATE) {
           v *= sigmoid_f32(p.epi_ptr[s * p.epi_rs + z]);
+        } else if constexpr (EPI == EPI_ACT) {
+          v = unary_act(v, p.act, p.epi_ptr, p.epi_c);
         }
         st_f32<TO>(O + s * p.out_rs + n, v);
       }
@@ -306,6 +321,7 @@ int launch_tile(const LinArgs& p, int epi, int batch, hipStream_t s) {
   if (epi == EPI_GLU) linear_tile_kernel<TO, EPI_GLU><<<dim3((p.N + 63) / 64, my, batch), dim3(256), 0, s>>>(p);
   else if (epi == EPI_NONE) linear_tile_kernel<TO, EPI_NONE><<<dim3((p.N + 127) / 128, my, batch), dim3(256), 0, s>>>(p);
   else if (epi == EPI_SOFTCAP) linear_tile_kernel<TO, EPI_SOFTCAP><<<dim3((p.N + 127) / 128, my, batch), dim3(256), 0, s>>>(p);
+  else if (epi == EPI_ACT) linear_tile_kernel<TO, EPI_ACT><<<dim3((p.N + 127) / 128, my, batch), dim3(256), 0, s>>>(p);
   else linear_tile_kernel<TO, EPI_ROW_GATE><<<dim3((p.N + 127) / 128, my, batch), dim3(256), 0, s>>>(p);
   return 0;
 }
@@ -402,6 +418,8 @@ __global__ __launch_bounds__(256) void linear_fewrow_kernel(LinArgs p) {
         v = p.epi_c * tanhf(v / p.epi_c);
       } else if constexpr (EPI == EPI_ROW_GATE) {
         v *= sigmoid_f32(p.epi_ptr[s * p.epi_rs + z]);
+      } else if constexpr (EPI == EPI_ACT) {
+        v = unary_act(v, p.act, p.epi_ptr, p.epi_c);
       }
       st_f32<TO>(O + s * p.out_rs + n, v);
     }
@@ -414,6 +432,7 @@ int launch_fewrow(const LinArgs& p, int epi, dim3 grid, hipStream_t s) {
     case EPI_NONE: linear_fewrow_kernel<T, TO, EPI_NONE, NSUB><<<grid, dim3(256), 0, s>>>(p); break;
     case EPI_GLU: linear_fewrow_kernel<T, TO, EPI_GLU, NSUB><<<grid, dim3(256), 0, s>>>(p); break;
     case EPI_SOFTCAP: linear_fewrow_kernel<T, TO, EPI_SOFTCAP, NSUB><<<grid, dim3(256), 0, s>>>(p); break;
+    case EPI_ACT: linear_fewrow_kernel<T, TO, EPI_ACT, NSUB><<<grid, dim3(256), 0, s>>>(p); break;
     default: linear_fewrow_kernel<T, TO, EPI_ROW_GATE, NSUB><<<grid, dim3(256), 0, s>>>(p); break;
   }
   return 0;
@@ -436,6 +455,7 @@ int launch_epi(const LinArgs& p, int epi, dim3 grid, hipStream_t s) {
     case EPI_NONE: linear_kernel<T, TO, EPI_NONE><<<grid, dim3(256), 0, s>>>(p); break;
     case EPI_GLU: linear_kernel<T, TO, EPI_GLU><<<grid, dim3(256), 0, s>>>(p); break;
     case EPI_SOFTCAP: linear_kernel<T, TO, EPI_SOFTCAP><<<grid, dim3(256), 0, s>>>(p); break;
+    case EPI_ACT: linear_kernel<T, TO, EPI_ACT><<<grid, dim3(256), 0, s>>>(p); break;
     default: linear_kernel<T, TO, EPI_ROW_GATE><<<grid, dim3(256), 0, s>>>(p); break;
   }
   return 0;
@@ -453,7 +473,8 @@ extern "C" int nv_linear(const void* a, int64_t a_row_stride, const int32_t* a_r
   NV_CHECK_ARG(out_dtype == NV_BF16 || out_dtype == NV_F32, "nv_linear: bad output dtype %d", out_dtype);
   NV_CHECK_ARG(M >= 0 && N > 0 && K > 0 && batch > 0 && batch <= 65535, "nv_linear: bad shape M=%lld N=%d K=%d batch=%d",
                (long long)M, N, K, batch);
-  NV_CHECK_ARG(epilogue >= EPI_NONE && epilogue <= EPI_ROW_GATE, "nv_linear: bad epilogue %d", epilogue);
+  NV_CHECK_ARG(epilogue >= EPI_NONE && epilogue <= EPI_ACT, "nv_linear: bad epilogue %d", epilogue);
+  NV_CHECK_ARG(epilogue != EPI_ACT || (act >= 0 && act <= 3 && (act != 2 || epi_ptr)), "nv_linear: bad activation %d", act);
   NV_CHECK_ARG(epilogue != EPI_ROW_GATE || epi_ptr, "nv_linear: the row-gate epilogue needs its gate rows");
   NV_CHECK_ARG(epilogue != EPI_SOFTCAP || epi_const > 0.0f, "nv_linear: the soft cap must be positive");
   if (M == 0) return NV_OK;

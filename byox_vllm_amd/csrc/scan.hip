@@ -1,0 +1,282 @@
+// Recurrences with an fp32 state per request, and the short causal convolution that feeds them.  All of them walk the
+// tokens a step brings for a request in order, starting from the request's slot (or from zero when the request has no
+// tokens behind it) and leaving the state there, so a prompt, its portions and single decoded tokens go one way.
+//
+// causal_conv:  out[t][c] = act(bias[c] + sum_j w[c][j] * x[t - (taps - 1 - j)][c]); the slot keeps the last
+//               taps - 1 inputs of every channel.
+// rglru_scan:   a = exp(-c * sigmoid(gr) * softplus(lam)),  S = a S + sqrt(1 - a^2) * sigmoid(gi) * u,
+//               out = S * gelu_tanh(y) * out_scale: the real-gated linear recurrent unit of the Griffin block.
+// ssd_scan:     per head, S [N, P]:  S = exp(-exp(A_log) dt) S + dt B x^T,  y = S^T C + D x,  dt = softplus(raw + bias);
+//               out = y * silu(z): the selective state-space recurrence of Mamba-2 in its token-by-token form.
+#include "anyt.h"
+
+namespace {
+
+constexpr int CONV_MAX_TAPS = 8;
+
+__device__ __forceinline__ float softplus_f32(float z) { return fmaxf(z, 0.0f) + log1pf(expf(-fabsf(z))); }
+
+struct ConvArgs {
+  const float* x;         // [tokens, x_rs] inputs (fp32 projections, bias included)
+  int64_t x_rs;
+  const void* w;          // [C, taps]
+  const void* bias;       // [C] or null
+  float* state;           // [slots, taps - 1, C]
+  const int32_t* cu_q;
+  const int32_t* past;
+  const int32_t* slots;
+  const int32_t* seq_of;
+  float* out_f32;         // [tokens, of_rs] or null
+  int64_t of_rs;
+  void* out_t;            // [tokens, ot_rs] in the storage type, or null
+  int64_t ot_rs;
+  int C, taps, act;       // act 0: none, 1: SiLU
+};
+
+// One thread per (token, channel).  Only a portion's first taps - 1 tokens need the slot; they are all served by the
+// thread of the portion's FIRST token, which afterwards writes the slot's new contents: every access to a slot's
+// channel comes from one thread, in program order.
+template <typename T>
+__global__ __launch_bounds__(256) void causal_conv_kernel(ConvArgs p) {
+  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  const int64_t t = blockIdx.x;
+  if (c >= p.C) return;
+  const int b = p.seq_of[t];
+  const int64_t t0 = p.cu_q[b];
+  const int k = (int)(t - t0), taps = p.taps, keep = taps - 1;
+  if (k > 0 && k < keep) return;
+  const T* w = reinterpret_cast<const T*>(p.w) + (int64_t)c * taps;
+  const float bias = p.bias ? ld_f32<T>(reinterpret_cast<const T*>(p.bias) + c) : 0.0f;
+  float wt[CONV_MAX_TAPS];
+#pragma unroll
+  for (int j = 0; j < CONV_MAX_TAPS; ++j) wt[j] = j < taps ? ld_f32<T>(w + j) : 0.0f;
+  auto emit = [&](int64_t tt, float v) {
+    if (p.act == 1) v = silu_f32(v);
+    if (p.out_f32) p.out_f32[tt * p.of_rs + c] = v;
+    if (p.out_t) st_f32<T>(reinterpret_cast<T*>(p.out_t) + tt * p.ot_rs + c, v);
+  };
+  if (k >= keep) {
+    float v = bias;
+#pragma unroll
+    for (int j = 0; j < CONV_MAX_TAPS; ++j)
+      if (j < taps) v += wt[j] * p.x[(t - (keep - j)) * p.x_rs + c];
+    emit(t, v);
+    return;
+  }
+  // k == 0: the tokens that reach back over the portion's start
+  const int n = p.cu_q[b + 1] - (int)t0;
+  float* slot = p.state + (int64_t)p.slots[b] * keep * p.C;
+  const bool fresh = p.past[b] == 0;
+  float st[CONV_MAX_TAPS];
+#pragma unroll
+  for (int i = 0; i < CONV_MAX_TAPS; ++i) st[i] = (i < keep && !fresh) ? slot[(int64_t)i * p.C + c] : 0.0f;
+  const int head = min(keep, n);
+  for (int kk = 0; kk < head; ++kk) {
+    float v = bias;
+#pragma unroll
+    for (int j = 0; j < CONV_MAX_TAPS; ++j) {
+      if (j >= taps) continue;
+      const int src = kk - (keep - j);
+      v += wt[j] * (src >= 0 ? p.x[(t0 + src) * p.x_rs + c] : st[kk + j]);
+    }
+    emit(t0 + kk, v);
+  }
+#pragma unroll
+  for (int i = 0; i < CONV_MAX_TAPS; ++i) {
+    if (i >= keep) continue;
+    const int src = n - keep + i;
+    slot[(int64_t)i * p.C + c] = src >= 0 ? p.x[(t0 + src) * p.x_rs + c] : st[i + n];
+  }
+}
+
+struct RglruArgs {
+  const float* u;         // [tokens, u_rs] convolution output
+  int64_t u_rs;
+  const float* gates;     // [tokens, g_rs]: per block of bw channels, bw recurrence-gate logits then bw input-gate logits
+  int64_t g_rs;
+  const float* y;         // [tokens, y_rs] the other branch before its activation
+  int64_t y_rs;
+  const void* lam;        // [C]
+  float* state;           // [slots, C]
+  const int32_t* cu_q;
+  const int32_t* past;
+  const int32_t* slots;
+  void* out;              // [tokens, out_rs]
+  int64_t out_rs;
+  int C, bw;
+  float c, out_scale;
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void rglru_scan_kernel(RglruArgs p) {
+  const int ch = blockIdx.x * blockDim.x + threadIdx.x;
+  const int b = blockIdx.y;
+  if (ch >= p.C) return;
+  const int t0 = p.cu_q[b], t1 = p.cu_q[b + 1];
+  if (t1 <= t0) return;
+  float* slot = p.state + (int64_t)p.slots[b] * p.C + ch;
+  float S = p.past[b] == 0 ? 0.0f : *slot;
+  const float sp = p.c * softplus_f32(ld_f32<T>(reinterpret_cast<const T*>(p.lam) + ch));
+  const int gcol = (ch / p.bw) * 2 * p.bw + ch % p.bw;
+  T* out = reinterpret_cast<T*>(p.out);
+  for (int64_t t = t0; t < t1; ++t) {
+    const float gr = p.gates[t * p.g_rs + gcol], gi = p.gates[t * p.g_rs + gcol + p.bw];
+    const float log_a = -sp * sigmoid_f32(gr);
+    // sqrt(1 - a^2) through expm1: 1 - exp(2 log a) loses its digits when the decay is close to one
+    S = expf(log_a) * S + sqrtf(-expm1f(2.0f * log_a)) * sigmoid_f32(gi) * p.u[t * p.u_rs + ch];
+    st_f32<T>(out + t * p.out_rs + ch, S * gelu_tanh_f32(p.y[t * p.y_rs + ch]) * p.out_scale);
+  }
+  *slot = S;
+}
+
+struct SsdArgs {
+  const float* xbc;       // [tokens, xbc_rs]: x (H * P) | B (G * N) | C (G * N), after convolution and activation
+  int64_t xbc_rs;
+  const float* z;         // [tokens, z_rs] gate, H * P
+  int64_t z_rs;
+  const float* dt;        // [tokens, dt_rs] raw step sizes, H
+  int64_t dt_rs;
+  const void* dt_bias;    // [H]
+  const void* A_log;      // [H]
+  const void* D;          // [H]
+  float* state;           // [slots, H, N, P]
+  const int32_t* cu_q;
+  const int32_t* past;
+  const int32_t* slots;
+  float* out;             // [tokens, H * P]
+  int H, G, N, P, parts;
+};
+
+// One workgroup per (request, head); thread (part, v) keeps S[part + parts * i][v], i < DPT, in registers.
+template <typename T, int DPT>
+__global__ __launch_bounds__(1024) void ssd_scan_kernel(SsdArgs p) {
+  extern __shared__ float lds[];
+  float* sB = lds;                    // [N] dt * B
+  float* sC = sB + p.N;               // [N]
+  float* so = sC + p.N;               // [parts][P]
+  const int h = blockIdx.x, b = blockIdx.y;
+  const int tid = threadIdx.x;
+  const bool active = tid < p.parts * p.P;
+  const int v = tid % p.P, part = tid / p.P;
+  const int t0 = p.cu_q[b], t1 = p.cu_q[b + 1];
+  if (t1 <= t0) return;
+  const int grp = h / (p.H / p.G);
+  float* S_g = p.state + ((int64_t)p.slots[b] * p.H + h) * p.N * p.P;
+  const bool fresh = p.past[b] == 0;
+  float S[DPT];
+#pragma unroll
+  for (int i = 0; i < DPT; ++i) {
+    const int n = part + p.parts * i;
+    S[i] = (active && n < p.N && !fresh) ? S_g[(int64_t)n * p.P + v] : 0.0f;
+  }
+  const float rate = expf(ld_f32<T>(reinterpret_cast<const T*>(p.A_log) + h));
+  const float dtb = ld_f32<T>(reinterpret_cast<const T*>(p.dt_bias) + h);
+  const float Dh = ld_f32<T>(reinterpret_cast<const T*>(p.D) + h);
+  const int inner = p.H * p.P;
+  for (int64_t t = t0; t < t1; ++t) {
+    const float* row = p.xbc + t * p.xbc_rs;
+    const float dt = softplus_f32(p.dt[t * p.dt_rs + h] + dtb);
+    const float decay = expf(-rate * dt);
+    for (int j = tid; j < p.N; j += blockDim.x) {
+      sB[j] = dt * row[inner + grp * p.N + j];
+      sC[j] = row[inner + p.G * p.N + grp * p.N + j];
+    }
+    const float xv = active ? row[h * p.P + v] : 0.0f;
+    __syncthreads();
+    float o = 0.0f;
+#pragma unroll
+    for (int i = 0; i < DPT; ++i) {
+      const int n = part + p.parts * i;
+      if (n < p.N) {
+        S[i] = decay * S[i] + sB[n] * xv;
+        o += S[i] * sC[n];
+      }
+    }
+    if (active) so[part * p.P + v] = o;
+    __syncthreads();
+    if (tid < p.P) {
+      float y = 0.0f;
+      for (int q = 0; q < p.parts; ++q) y += so[q * p.P + tid];
+      y += Dh * row[h * p.P + tid];
+      p.out[t * inner + h * p.P + tid] = y * silu_f32(p.z[t * p.z_rs + h * p.P + tid]);
+    }
+  }
+  if (active) {
+#pragma unroll
+    for (int i = 0; i < DPT; ++i) {
+      const int n = part + p.parts * i;
+      if (n < p.N) S_g[(int64_t)n * p.P + v] = S[i];
+    }
+  }
+}
+
+}  // namespace
+
+extern "C" int nv_causal_conv(const float* x, int64_t x_row_stride, const void* w, const void* bias, float* state,
+                              const int32_t* cu_q, const int32_t* past_lens, const int32_t* state_slots,
+                              const int32_t* seq_of_token, float* out_f32, int64_t out_f32_row_stride, void* out_t,
+                              int64_t out_t_row_stride, int64_t tokens, int channels, int taps, int act, int dtype,
+                              nv_stream_t stream) {
+  NV_CHECK_ARG(x && w && state && cu_q && past_lens && state_slots && seq_of_token && (out_f32 || out_t),
+               "nv_causal_conv: null pointer");
+  NV_CHECK_ARG(dtype == NV_BF16 || dtype == NV_F32, "nv_causal_conv: bad dtype %d", dtype);
+  NV_CHECK_ARG(tokens >= 0 && tokens < (1ll << 31) && channels > 0 && taps >= 1 && taps <= CONV_MAX_TAPS &&
+                   (act == 0 || act == 1),
+               "nv_causal_conv: bad shape (taps up to %d)", CONV_MAX_TAPS);
+  if (tokens == 0) return NV_OK;
+  ConvArgs p{x, x_row_stride, w, bias, state, cu_q, past_lens, state_slots, seq_of_token, out_f32, out_f32_row_stride,
+             out_t, out_t_row_stride, channels, taps, act};
+  NV_DISPATCH_T(dtype, causal_conv_kernel<T><<<dim3((unsigned)tokens, (unsigned)((channels + 255) / 256)), dim3(256), 0,
+                                               (hipStream_t)stream>>>(p));
+  NV_CHECK_LAUNCH();
+  return NV_OK;
+}
+
+extern "C" int nv_rglru_scan(const float* u, int64_t u_row_stride, const float* gates, int64_t gates_row_stride,
+                             const float* y, int64_t y_row_stride, const void* lam, float* state, const int32_t* cu_q,
+                             const int32_t* past_lens, const int32_t* state_slots, void* out, int64_t out_row_stride,
+                             int num_seqs, int channels, int block_width, float c, float out_scale, int dtype,
+                             nv_stream_t stream) {
+  NV_CHECK_ARG(u && gates && y && lam && state && cu_q && past_lens && state_slots && out, "nv_rglru_scan: null pointer");
+  NV_CHECK_ARG(dtype == NV_BF16 || dtype == NV_F32, "nv_rglru_scan: bad dtype %d", dtype);
+  NV_CHECK_ARG(num_seqs >= 0 && num_seqs <= 65535 && channels > 0 && block_width > 0 && channels % block_width == 0,
+               "nv_rglru_scan: bad shape");
+  if (num_seqs == 0) return NV_OK;
+  RglruArgs p{u, u_row_stride, gates, gates_row_stride, y, y_row_stride, lam, state, cu_q, past_lens, state_slots, out,
+              out_row_stride, channels, block_width, c, out_scale};
+  const int threads = 64;
+  NV_DISPATCH_T(dtype, rglru_scan_kernel<T><<<dim3((unsigned)((channels + threads - 1) / threads), (unsigned)num_seqs),
+                                              dim3(threads), 0, (hipStream_t)stream>>>(p));
+  NV_CHECK_LAUNCH();
+  return NV_OK;
+}
+
+extern "C" int nv_ssd_scan(const float* xbc, int64_t xbc_row_stride, const float* z, int64_t z_row_stride, const float* dt,
+                           int64_t dt_row_stride, const void* dt_bias, const void* A_log, const void* D, float* state,
+                           const int32_t* cu_q, const int32_t* past_lens, const int32_t* state_slots, float* out,
+                           int num_seqs, int heads, int groups, int state_size, int vdim, int dtype, nv_stream_t stream) {
+  NV_CHECK_ARG(xbc && z && dt && dt_bias && A_log && D && state && cu_q && past_lens && state_slots && out,
+               "nv_ssd_scan: null pointer");
+  NV_CHECK_ARG(dtype == NV_BF16 || dtype == NV_F32, "nv_ssd_scan: bad dtype %d", dtype);
+  NV_CHECK_ARG(num_seqs >= 0 && num_seqs <= 65535 && heads > 0 && groups > 0 && heads % groups == 0 && state_size > 0 &&
+                   vdim > 0 && vdim <= 1024,
+               "nv_ssd_scan: bad shape");
+  if (num_seqs == 0) return NV_OK;
+  // threads: vdim columns times `parts` slices of the state rows; each thread keeps up to DPT rows of its column
+  int parts = 1024 / vdim;
+  if (parts > state_size) parts = state_size;
+  if (parts > 8) parts = 8;
+  const int per = (state_size + parts - 1) / parts;
+  NV_CHECK_ARG(per <= 64, "nv_ssd_scan: a state of %d x %d exceeds one workgroup's registers", state_size, vdim);
+  SsdArgs p{xbc, xbc_row_stride, z, z_row_stride, dt, dt_row_stride, dt_bias, A_log, D, state, cu_q, past_lens,
+            state_slots, out, heads, groups, state_size, vdim, parts};
+  const int threads = ((parts * vdim + 63) / 64) * 64;
+  const size_t lds = (size_t)(2 * state_size + parts * vdim) * sizeof(float);
+  dim3 grid((unsigned)heads, (unsigned)num_seqs);
+  hipStream_t s = (hipStream_t)stream;
+  if (per <= 4) NV_DISPATCH_T(dtype, ssd_scan_kernel<T, 4><<<grid, dim3(threads), lds, s>>>(p));
+  else if (per <= 16) NV_DISPATCH_T(dtype, ssd_scan_kernel<T, 16><<<grid, dim3(threads), lds, s>>>(p));
+  else NV_DISPATCH_T(dtype, ssd_scan_kernel<T, 64><<<grid, dim3(threads), lds, s>>>(p));
+  NV_CHECK_LAUNCH();
+  return NV_OK;
+}

@@ -1,0 +1,227 @@
+// Softmax attention over a paged cache with grouped key/value heads, key and value sizes that may differ, and a score
+// that is shaped before the softmax:
+//     s_ij = cap(q_i . k_j) - slope_h (i - j),   cap(z) = c tanh(z / c) (or z without a cap),
+// over the keys 0 <= i - j < window (window 0: every earlier key).  q arrives already normalised and multiplied by its
+// scale and per-head temperature (qk_norm_store below), so the kernel's own arithmetic is the dot product, the cap,
+// the distance term and the softmax, all in fp32.
+//
+// qk_norm_store: per token, RMS norm over each query and key head (one weight vector shared by the heads), the query
+// scaled by scale * temp[h] and left in fp32, the normalised key and the value written to the token's cache row
+// [k: G * d | v: G * dv] in the storage type.
+//
+// window_attn_kernel: a workgroup owns TQ consecutive tokens of the packed batch and one key/value head, i.e. up to
+// TQ * (H / G) query rows that read the same keys; tokens of different requests inside the tile are served one request
+// after the other.  Keys go through LDS in tiles of TK rows; online softmax per row.
+#include "anyt.h"
+
+namespace {
+
+struct QkArgs {
+  const float* proj;      // [tokens, proj_rs]: q | k | v at the given column offsets (fp32 projections, bias included)
+  int64_t proj_rs;
+  int q_off, k_off, v_off;
+  const void* qn;         // [d] query norm weight
+  const void* kn;         // [d]
+  const void* temp;       // [H] or null
+  const int32_t* slot_mapping;   // [tokens] cache row of each token, -1: none
+  void* cache;            // [rows, G * (d + dv)]
+  float* q_out;           // [tokens, H * d]
+  int H, G, d, dv;
+  float scale, eps;
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void qk_norm_store_kernel(QkArgs p) {
+  const int64_t t = blockIdx.x;
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  const float* row = p.proj + t * p.proj_rs;
+  const int64_t slot = p.slot_mapping[t];
+  const int cw = p.G * (p.d + p.dv);
+  T* crow = slot >= 0 ? reinterpret_cast<T*>(p.cache) + slot * cw : nullptr;
+  const T* qn = reinterpret_cast<const T*>(p.qn);
+  const T* kn = reinterpret_cast<const T*>(p.kn);
+  const T* temp = reinterpret_cast<const T*>(p.temp);
+  for (int v = wv; v < p.H + p.G; v += nw) {
+    const bool is_q = v < p.H;
+    const float* src = is_q ? row + p.q_off + v * p.d : row + p.k_off + (v - p.H) * p.d;
+    float ss = 0.0f;
+    for (int e = lane; e < p.d; e += 64) ss += src[e] * src[e];
+    ss = wave_sum(ss);
+    const float inv = 1.0f / sqrtf(ss / (float)p.d + p.eps);
+    if (is_q) {
+      const float f = p.scale * (temp ? ld_f32<T>(temp + v) : 1.0f);
+      for (int e = lane; e < p.d; e += 64) p.q_out[t * p.H * p.d + v * p.d + e] = src[e] * inv * ld_f32<T>(qn + e) * f;
+    } else if (crow) {
+      for (int e = lane; e < p.d; e += 64) st_f32<T>(crow + (v - p.H) * p.d + e, src[e] * inv * ld_f32<T>(kn + e));
+    }
+  }
+  if (crow)
+    for (int e = threadIdx.x; e < p.G * p.dv; e += blockDim.x) st_f32<T>(crow + p.G * p.d + e, row[p.v_off + e]);
+}
+
+struct WAttnArgs {
+  const float* q;          // [tokens, H * d]
+  const void* cache;       // [rows, G * (d + dv)]
+  const int32_t* tables;   // [B, table_cols]
+  int table_cols;
+  const int32_t* cu_q;     // [B + 1]
+  const int32_t* past;     // [B]
+  const int32_t* seq_of;   // [tokens]
+  void* out;               // [tokens, out_rs]: head h at columns h * dv
+  int64_t out_rs;
+  int64_t tokens;
+  int H, G, d, dv, block_size, window, TQ, TK;
+  float softcap, out_scale;
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void window_attn_kernel(WAttnArgs p) {
+  extern __shared__ float lds[];
+  const int R = p.H / p.G, d = p.d, dv = p.dv, TK = p.TK, dp = d + 1;
+  const int maxrows = p.TQ * R;
+  float* sq = lds;                       // [rows][d]
+  float* sk = sq + maxrows * d;          // [TK][d + 1]
+  float* sv = sk + TK * dp;              // [TK][dv]
+  float* sc = sv + TK * dv;              // [rows][TK]
+  float* acc = sc + maxrows * TK;        // [rows][dv]
+  float* sm = acc + maxrows * dv;        // [rows] running maximum
+  float* sl = sm + maxrows;              // [rows] running sum
+  float* scorr = sl + maxrows;           // [rows]
+  const int g = blockIdx.y;
+  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  const int64_t t_begin = (int64_t)blockIdx.x * p.TQ;
+  const int64_t t_end = min(p.tokens, t_begin + p.TQ);
+  const T* cache = reinterpret_cast<const T*>(p.cache);
+  const int cw = p.G * (d + dv);
+  T* out = reinterpret_cast<T*>(p.out);
+
+  for (int64_t ts = t_begin; ts < t_end;) {
+    const int b = p.seq_of[ts];
+    const int64_t te = min(t_end, (int64_t)p.cu_q[b + 1]);
+    const int nq = (int)(te - ts), rows = nq * R;
+    const int p0 = p.past[b] + (int)(ts - p.cu_q[b]);
+    const int32_t* table = p.tables + (int64_t)b * p.table_cols;
+    for (int i = tid; i < rows * d; i += 256) {
+      const int rr = i / d, e = i % d;
+      sq[i] = p.q[(ts + rr / R) * p.H * d + (g * R + rr % R) * d + e];
+    }
+    for (int i = tid; i < rows * dv; i += 256) acc[i] = 0.0f;
+    if (tid < rows) {
+      sm[tid] = -INFINITY;
+      sl[tid] = 0.0f;
+    }
+    __syncthreads();
+    const int lo = p.window > 0 ? max(0, p0 - p.window + 1) : 0, hi = p0 + nq - 1;
+    for (int j0 = lo; j0 <= hi; j0 += TK) {
+      const int nk = min(TK, hi + 1 - j0);
+      for (int i = tid; i < nk * (d + dv); i += 256) {
+        const int j = i / (d + dv), e = i % (d + dv);
+        const int kp = j0 + j;
+        const int64_t crow = (int64_t)table[kp / p.block_size] * p.block_size + kp % p.block_size;
+        if (e < d) sk[j * dp + e] = ld_f32<T>(cache + crow * cw + g * d + e);
+        else sv[j * dv + e - d] = ld_f32<T>(cache + crow * cw + p.G * d + g * dv + e - d);
+      }
+      __syncthreads();
+      for (int i = tid; i < rows * TK; i += 256) {
+        const int rr = i / TK, j = i % TK;
+        const int pos = p0 + rr / R, kp = j0 + j;
+        float s = -INFINITY;
+        if (j < nk && kp <= pos && (p.window <= 0 || pos - kp < p.window)) {
+          s = 0.0f;
+          const float* qv = sq + rr * d;
+          const float* kv = sk + j * dp;
+          for (int e = 0; e < d; ++e) s += qv[e] * kv[e];
+          if (p.softcap > 0.0f) s = p.softcap * tanhf(s / p.softcap);
+          const int h = g * R + rr % R;
+          s -= exp2f(-8.0f * (float)(h + 1) / (float)p.H) * (float)(pos - kp);
+        }
+        sc[i] = s;
+      }
+      __syncthreads();
+      for (int rr = wv; rr < rows; rr += 4) {
+        float m = -INFINITY;
+        for (int j = lane; j < TK; j += 64) m = fmaxf(m, sc[rr * TK + j]);
+        m = wave_max(m);
+        const float m_old = sm[rr];
+        const float m_new = fmaxf(m_old, m);
+        float sum = 0.0f;
+        for (int j = lane; j < TK; j += 64) {
+          const float s = sc[rr * TK + j];
+          const float e = s == -INFINITY ? 0.0f : expf(s - m_new);
+          sc[rr * TK + j] = e;
+          sum += e;
+        }
+        sum = wave_sum(sum);
+        if (lane == 0) {
+          const float corr = m_new == -INFINITY ? 1.0f : expf(m_old - m_new);   // exp(-inf) = 0 at the first tile
+          scorr[rr] = corr;
+          sm[rr] = m_new;
+          sl[rr] = sl[rr] * corr + sum;
+        }
+      }
+      __syncthreads();
+      for (int i = tid; i < rows * dv; i += 256) {
+        const int rr = i / dv, e = i % dv;
+        float a = acc[i] * scorr[rr];
+        const float* pv = sc + rr * TK;
+        for (int j = 0; j < nk; ++j) a += pv[j] * sv[j * dv + e];
+        acc[i] = a;
+      }
+      __syncthreads();
+    }
+    for (int i = tid; i < rows * dv; i += 256) {
+      const int rr = i / dv, e = i % dv;
+      st_f32<T>(out + (ts + rr / R) * p.out_rs + (g * R + rr % R) * dv + e, acc[i] / sl[rr] * p.out_scale);
+    }
+    __syncthreads();
+    ts = te;
+  }
+}
+
+}  // namespace
+
+extern "C" int nv_qk_norm_store(const float* proj, int64_t proj_row_stride, int q_off, int k_off, int v_off,
+                                const void* q_norm, const void* k_norm, const void* temp, float scale, float eps,
+                                const int32_t* slot_mapping, void* cache, float* q_out, int64_t tokens, int heads,
+                                int kv_heads, int dim, int vdim, int dtype, nv_stream_t stream) {
+  NV_CHECK_ARG(proj && q_norm && k_norm && slot_mapping && cache && q_out, "nv_qk_norm_store: null pointer");
+  NV_CHECK_ARG(dtype == NV_BF16 || dtype == NV_F32, "nv_qk_norm_store: bad dtype %d", dtype);
+  NV_CHECK_ARG(tokens >= 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && dim > 0 && vdim > 0,
+               "nv_qk_norm_store: bad shape");
+  if (tokens == 0) return NV_OK;
+  QkArgs p{proj, proj_row_stride, q_off, k_off, v_off, q_norm, k_norm, temp, slot_mapping, cache, q_out, heads, kv_heads,
+           dim, vdim, scale, eps};
+  NV_DISPATCH_T(dtype, qk_norm_store_kernel<T><<<dim3((unsigned)tokens), dim3(256), 0, (hipStream_t)stream>>>(p));
+  NV_CHECK_LAUNCH();
+  return NV_OK;
+}
+
+extern "C" int nv_window_attn(const float* q, const void* cache, const int32_t* block_tables, int table_cols,
+                              const int32_t* cu_q, const int32_t* past_lens, const int32_t* seq_of_token, void* out,
+                              int64_t out_row_stride, int64_t tokens, int max_q, int heads, int kv_heads, int dim, int vdim,
+                              int block_size, int window, float softcap, float out_scale, int dtype, nv_stream_t stream) {
+  NV_CHECK_ARG(q && cache && block_tables && cu_q && past_lens && seq_of_token && out, "nv_window_attn: null pointer");
+  NV_CHECK_ARG(dtype == NV_BF16 || dtype == NV_F32, "nv_window_attn: bad dtype %d", dtype);
+  NV_CHECK_ARG(tokens >= 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && dim > 0 && vdim > 0 &&
+                   block_size > 0 && window >= 0 && table_cols > 0,
+               "nv_window_attn: bad shape");
+  if (tokens == 0) return NV_OK;
+  const int R = heads / kv_heads;
+  const size_t budget = 64 * 1024;
+  auto need = [&](int tq, int tk) {
+    const size_t rows = (size_t)tq * R;
+    return (rows * dim + (size_t)tk * (dim + 1) + (size_t)tk * vdim + rows * tk + rows * vdim + 3 * rows) * sizeof(float);
+  };
+  int TQ = max_q <= 1 ? 1 : 16, TK = 64;
+  while (TK > 8 && need(1, TK) > budget) TK /= 2;
+  NV_CHECK_ARG(need(1, TK) <= budget, "nv_window_attn: heads of %d + %d numbers do not fit the LDS plan", dim, vdim);
+  while (TQ > 1 && (need(TQ, TK) > budget || TQ * R > 256)) TQ /= 2;
+  NV_CHECK_ARG(R <= 256 && kv_heads <= 65535, "nv_window_attn: %d query heads per key head exceed a workgroup", R);
+  const int64_t tiles = (tokens + TQ - 1) / TQ;
+  WAttnArgs p{q, cache, block_tables, table_cols, cu_q, past_lens, seq_of_token, out, out_row_stride, tokens, heads,
+              kv_heads, dim, vdim, block_size, window, TQ, TK, softcap, out_scale};
+  dim3 grid((unsigned)tiles, (unsigned)kv_heads);
+  NV_DISPATCH_T(dtype, window_attn_kernel<T><<<grid, dim3(256), need(TQ, TK), (hipStream_t)stream>>>(p));
+  NV_CHECK_LAUNCH();
+  return NV_OK;
+}

@@ -436,8 +436,8 @@ def stage_decode_packed(packed, bs, bt_cols, g, prev_tokens=None, block_size=0):
 # ---------------------------------------------------------------------------------------------------------------
 # Kernels of models with an fp32 residual stream (bf16 or true fp32 storage): nv_linear and its row-wise companions.
 
-EPI_NONE, EPI_GLU, EPI_SOFTCAP, EPI_ROW_GATE = 0, 1, 2, 3
-ACT_SILU, ACT_GELU_TANH = 0, 1
+EPI_NONE, EPI_GLU, EPI_SOFTCAP, EPI_ROW_GATE, EPI_ACT = 0, 1, 2, 3, 4
+ACT_SILU, ACT_GELU_TANH, ACT_XIELU, ACT_SCALE = 0, 1, 2, 3
 
 
 def _code32(dt) -> int:
@@ -641,4 +641,156 @@ def moe_combine(y, slot_of, weights, shared=None, shared_gate=None, out=None):
     check(lib().nv_moe_combine(ptr(y), ptr(slot_of), ptr(weights), top, ptr(shared), ptr(shared_gate),
                                shared_gate.stride(0) if shared_gate is not None else 0, ptr(out), T, width, stream()),
           "nv_moe_combine")
+    return out
+
+
+# ---- residual streams, token shift, shaped-score attention, recurrences with state slots ----
+def embed_sinusoid(ids, positions, table, inv_freq, streams, out=None):
+    """fp32 streams [T, streams, width], each table[id] + (sin, cos) pairs of position * inv_freq (float64 [ceil(width/2)])."""
+    require_gpu(table, "embed_sinusoid")
+    T, width = ids.numel(), table.size(1)
+    assert ids.dtype == positions.dtype == torch.int64 and ids.is_contiguous() and positions.is_contiguous()
+    assert positions.numel() == T and table.is_contiguous()
+    assert inv_freq.dtype == torch.float64 and inv_freq.is_cuda and inv_freq.numel() * 2 >= width
+    out = torch.empty(T, streams, width, dtype=torch.float32, device=table.device) if out is None else out
+    check(lib().nv_embed_sinusoid(ptr(ids), ptr(positions), ptr(table), ptr(inv_freq), ptr(out), T, streams, width,
+                                  table.size(0), _code32(table.dtype), stream()), "nv_embed_sinusoid")
+    return out
+
+
+def hc_norm(x, w, eps, hc_in=None, delta=None, hc_prev=None, rows_idx=None, one_plus=True, out_dtype=None, out=None):
+    """RMS norm of a weighted sum of the fp32 streams ``x`` [T, S, width].  ``delta`` [T, width] (the previous sublayer's
+    output) is first folded into the streams with ``hc_prev`` = in | out | mix of that sublayer (None: added to every
+    stream); ``hc_in`` [S] weighs the streams (None: their sum).  ``rows_idx`` gathers rows and leaves ``x`` alone."""
+    require_gpu(x, "hc_norm")
+    T, S, width = x.shape
+    assert x.dtype == torch.float32 and x.is_contiguous() and w.numel() == width and w.is_contiguous()
+    if delta is not None:
+        assert delta.dtype == torch.float32 and delta.stride(1) == 1 and delta.shape == (T, width)
+    for t, n in ((hc_prev, 2 * S + S * S), (hc_in, S)):
+        assert t is None or (t.dtype == torch.float32 and t.is_contiguous() and t.numel() >= n and t.is_cuda)
+    rows = T if rows_idx is None else rows_idx.numel()
+    if rows_idx is not None:
+        assert rows_idx.dtype == torch.int32
+    out_dtype = out_dtype or w.dtype
+    out = torch.empty(rows, width, dtype=out_dtype, device=x.device) if out is None else out
+    assert out.dtype == out_dtype and out.stride(1) == 1
+    check(lib().nv_hc_norm(ptr(x), S, width, ptr(delta), delta.stride(0) if delta is not None else 0,
+                           ptr(hc_prev) if delta is not None else None, ptr(hc_in), ptr(w), int(one_plus), eps,
+                           ptr(rows_idx), ptr(out), out.stride(0), _code32(out_dtype), rows, _code32(w.dtype), stream()),
+          "nv_hc_norm")
+    return out
+
+
+def token_shift(h, mu, state, cu_q, past_lens, state_slots, seq_of_token, out=None):
+    """h fp32 [T, width] -> h + (previous row - h) * mu in the dtype of ``mu``; ``state`` fp32 [slots, width]."""
+    require_gpu(h, "token_shift")
+    T, width = h.shape
+    assert h.dtype == state.dtype == torch.float32 and h.is_contiguous() and state.is_contiguous()
+    assert state.size(-1) == width and mu.numel() == width
+    assert cu_q.dtype == past_lens.dtype == state_slots.dtype == seq_of_token.dtype == torch.int32
+    assert seq_of_token.numel() == T and cu_q.numel() == past_lens.numel() + 1 == state_slots.numel() + 1
+    out = torch.empty(T, width, dtype=mu.dtype, device=h.device) if out is None else out
+    check(lib().nv_token_shift(ptr(h), ptr(mu), ptr(state), ptr(cu_q), ptr(past_lens), ptr(state_slots),
+                               ptr(seq_of_token), ptr(out), T, width, _code32(mu.dtype), stream()), "nv_token_shift")
+    return out
+
+
+def group_rms_norm_f32(x, w, groups, eps, out=None):
+    """fp32 rows [T, groups * n]: every part of n numbers by its own root mean square, times w -> rows in w's dtype."""
+    require_gpu(x, "group_rms_norm_f32")
+    assert x.dim() == 2 and x.dtype == torch.float32 and x.stride(1) == 1 and w.numel() == x.size(1)
+    assert x.size(1) % groups == 0
+    out = torch.empty(x.shape, dtype=w.dtype, device=x.device) if out is None else out
+    check(lib().nv_group_rmsnorm_f32(ptr(x), x.stride(0), ptr(w), ptr(out), out.stride(0), x.size(0), groups,
+                                     x.size(1) // groups, eps, _code32(w.dtype), stream()), "nv_group_rmsnorm_f32")
+    return out
+
+
+def qk_norm_store(proj, offsets, q_norm, k_norm, temp, scale, eps, slot_mapping, cache, heads, kv_heads, dim, vdim):
+    """fp32 projections [T, *] with q | k | v at ``offsets`` -> fp32 queries [T, heads * dim] (normalised, times scale and
+    the head's temperature); normalised keys and values go to the cache rows [G * dim | G * vdim] of ``slot_mapping``."""
+    require_gpu(proj, "qk_norm_store")
+    T = proj.size(0)
+    assert proj.dtype == torch.float32 and proj.stride(1) == 1 and slot_mapping.dtype == torch.int32
+    assert slot_mapping.numel() == T and cache.is_contiguous() and cache.size(-1) == kv_heads * (dim + vdim)
+    assert q_norm.numel() == k_norm.numel() == dim and q_norm.dtype == k_norm.dtype == cache.dtype
+    assert temp is None or (temp.numel() == heads and temp.dtype == cache.dtype)
+    q_off, k_off, v_off = offsets
+    assert max(q_off + heads * dim, k_off + kv_heads * dim, v_off + kv_heads * vdim) <= proj.size(1)
+    q = torch.empty(T, heads * dim, dtype=torch.float32, device=proj.device)
+    check(lib().nv_qk_norm_store(ptr(proj), proj.stride(0), q_off, k_off, v_off, ptr(q_norm), ptr(k_norm), ptr(temp),
+                                 scale, eps, ptr(slot_mapping), ptr(cache), ptr(q), T, heads, kv_heads, dim, vdim,
+                                 _code32(cache.dtype), stream()), "nv_qk_norm_store")
+    return q
+
+
+def window_attn(q, cache, block_tables, cu_q, past_lens, seq_of_token, max_q, heads, kv_heads, dim, vdim, block_size,
+                window, softcap, out, out_scale=1.0):
+    """Attention of fp32 queries [T, heads * dim] over the paged cache; ``out`` [T, >= heads * vdim] (a column slice of a
+    wider buffer is fine) in the cache dtype receives out_scale * the weighted values."""
+    require_gpu(q, "window_attn")
+    T = q.size(0)
+    assert q.dtype == torch.float32 and q.is_contiguous() and q.size(1) == heads * dim and cache.is_contiguous()
+    assert block_tables.dtype == torch.int32 and block_tables.is_contiguous() and block_tables.dim() == 2
+    assert cu_q.dtype == past_lens.dtype == seq_of_token.dtype == torch.int32 and seq_of_token.numel() == T
+    assert out.dtype == cache.dtype and out.stride(1) == 1 and out.size(0) == T and out.size(1) >= heads * vdim
+    check(lib().nv_window_attn(ptr(q), ptr(cache), ptr(block_tables), block_tables.size(1), ptr(cu_q), ptr(past_lens),
+                               ptr(seq_of_token), ptr(out), out.stride(0), T, max_q, heads, kv_heads, dim, vdim,
+                               block_size, window, float(softcap or 0.0), out_scale, _code32(cache.dtype), stream()),
+          "nv_window_attn")
+    return out
+
+
+def causal_conv(x, w, bias, state, cu_q, past_lens, state_slots, seq_of_token, act=0, want_f32=True, want_t=False):
+    """Per-channel causal convolution of fp32 rows ``x`` [T, C] (a column slice is fine) with ``w`` [C, taps]; ``state``
+    fp32 [slots, taps - 1, C].  -> (fp32 result or None, result in w's dtype or None)."""
+    require_gpu(x, "causal_conv")
+    T, C = x.shape
+    taps = w.size(1)
+    assert x.dtype == state.dtype == torch.float32 and x.stride(1) == 1 and w.shape == (C, taps) and w.is_contiguous()
+    assert state.is_contiguous() and state.shape[1:] == (max(taps - 1, 0), C) and seq_of_token.numel() == T
+    assert bias is None or (bias.numel() == C and bias.dtype == w.dtype)
+    assert cu_q.dtype == past_lens.dtype == state_slots.dtype == seq_of_token.dtype == torch.int32
+    of = torch.empty(T, C, dtype=torch.float32, device=x.device) if want_f32 else None
+    ot = torch.empty(T, C, dtype=w.dtype, device=x.device) if want_t else None
+    check(lib().nv_causal_conv(ptr(x), x.stride(0), ptr(w), ptr(bias), ptr(state), ptr(cu_q), ptr(past_lens),
+                               ptr(state_slots), ptr(seq_of_token), ptr(of), C, ptr(ot), C, T, C, taps, act,
+                               _code32(w.dtype), stream()), "nv_causal_conv")
+    return of, ot
+
+
+def rglru_scan(u, gates, y, lam, state, cu_q, past_lens, state_slots, block_width, out, c=8.0, out_scale=1.0):
+    """Real-gated linear recurrence over fp32 rows u [T, C]; ``gates`` fp32 [T, 2C] (per block: recurrence-gate logits,
+    then input-gate logits); ``y`` fp32 [T, C] is the other branch before its GELU; ``state`` fp32 [slots, C];
+    ``out`` [T, >= C] in lam's dtype."""
+    require_gpu(u, "rglru_scan")
+    T, C = u.shape
+    assert u.dtype == gates.dtype == y.dtype == state.dtype == torch.float32
+    assert u.stride(1) == gates.stride(1) == y.stride(1) == out.stride(1) == 1 and gates.shape == (T, 2 * C)
+    assert y.shape == (T, C) and state.is_contiguous() and state.size(-1) == C and lam.numel() == C
+    assert out.dtype == lam.dtype and out.size(0) == T and out.size(1) >= C and C % block_width == 0
+    assert cu_q.dtype == past_lens.dtype == state_slots.dtype == torch.int32
+    check(lib().nv_rglru_scan(ptr(u), u.stride(0), ptr(gates), gates.stride(0), ptr(y), y.stride(0), ptr(lam), ptr(state),
+                              ptr(cu_q), ptr(past_lens), ptr(state_slots), ptr(out), out.stride(0), past_lens.numel(), C,
+                              block_width, c, out_scale, _code32(lam.dtype), stream()), "nv_rglru_scan")
+    return out
+
+
+def ssd_scan(xbc, z, dt, dt_bias, A_log, D, state, cu_q, past_lens, state_slots, heads, groups, state_size, vdim):
+    """Selective state-space recurrence over fp32 rows xbc [T, heads*vdim + 2*groups*state] -> fp32 [T, heads*vdim]
+    (already multiplied by silu(z)); ``state`` fp32 [slots, heads, state, vdim]."""
+    require_gpu(xbc, "ssd_scan")
+    T = xbc.size(0)
+    inner = heads * vdim
+    assert xbc.dtype == z.dtype == dt.dtype == state.dtype == torch.float32
+    assert xbc.stride(1) == z.stride(1) == dt.stride(1) == 1 and xbc.size(1) == inner + 2 * groups * state_size
+    assert z.shape == (T, inner) and dt.shape == (T, heads) and state.is_contiguous()
+    assert state.shape[1:] == (heads, state_size, vdim) and dt_bias.numel() == A_log.numel() == D.numel() == heads
+    assert dt_bias.dtype == A_log.dtype == D.dtype
+    assert cu_q.dtype == past_lens.dtype == state_slots.dtype == torch.int32
+    out = torch.empty(T, inner, dtype=torch.float32, device=xbc.device)
+    check(lib().nv_ssd_scan(ptr(xbc), xbc.stride(0), ptr(z), z.stride(0), ptr(dt), dt.stride(0), ptr(dt_bias), ptr(A_log),
+                            ptr(D), ptr(state), ptr(cu_q), ptr(past_lens), ptr(state_slots), ptr(out), past_lens.numel(),
+                            heads, groups, state_size, vdim, _code32(dt_bias.dtype), stream()), "nv_ssd_scan")
     return out

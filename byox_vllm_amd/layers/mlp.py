@@ -1,0 +1,38 @@
+"""Feed-forward with one up-projection and an element-wise activation, W_down act(W_up h); the activation runs in the
+up-projection's epilogue.  ``xielu`` is the activation with two learned numbers p, q:
+
+    z > 0:  softplus(p) z^2 + z / 2;        z <= 0:  (1/2 + softplus(q)) (exp(z) - 1 - z) + z / 2
+
+whose coefficients are evaluated once after loading (fp32, on the device) and read by the kernel."""
+
+import torch
+from torch import nn
+
+from byox_vllm_amd import kernels
+from byox_vllm_amd.layers.linear import DenseLinear
+
+UNARY = {"silu": kernels.ACT_SILU, "gelu_tanh": kernels.ACT_GELU_TANH, "xielu": kernels.ACT_XIELU}
+
+
+class UnaryMLP(nn.Module):
+    def __init__(self, width: int, ff: int, act: str):
+        super().__init__()
+        self.act = UNARY[act]
+        self.up = DenseLinear(width, ff)
+        self.down = DenseLinear(ff, width)
+        if act == "xielu":
+            self.act_params = nn.Parameter(torch.zeros(2, dtype=torch.float32), requires_grad=False)
+            self.act_params.weight_loader = lambda p, t: p.data.copy_(t.reshape(2).to(torch.float32))
+        self.coef = None
+
+    def finalize(self) -> None:
+        """The activation's coefficients from its stored numbers (softplus in float64, then fp32)."""
+        if self.act == kernels.ACT_XIELU:
+            sp = torch.nn.functional.softplus(self.act_params.data.to(torch.float64))
+            self.coef = torch.stack([sp[0], 0.5 + sp[1]]).to(torch.float32).contiguous()
+
+    def forward(self, h):
+        if self.act == kernels.ACT_XIELU and self.coef is None:
+            self.finalize()
+        hidden = self.up(h, epilogue=kernels.EPI_ACT, act=self.act, gate=self.coef)
+        return self.down(hidden, out_dtype=torch.float32)

@@ -9,6 +9,7 @@ _MODELS = {
     "Qwen2ForCausalLM": ("byox_vllm_amd.models.qwen3", "Qwen3ForCausalLM"),
     "Qwen3ForCausalLM": ("byox_vllm_amd.models.qwen3", "Qwen3ForCausalLM"),
     "Rurutar": ("byox_vllm_amd.models.rurutar", "RurutarForCausalLM"),
+    "Nonetar": ("byox_vllm_amd.models.nonetar", "NonetarForCausalLM"),
 }
 DEFAULT = "Qwen3ForCausalLM"
 

@@ -340,6 +340,8 @@ int nv_gemm_lt_f32out(const void* x, int64_t x_row_stride, const void* w_rowmajo
  *   epilogue     0 none; 1 gated unit: W holds N gate rows followed by N up rows, out = act(gate) * up with act = SiLU
  *                (act 0) or the tanh form of GELU (act 1); 2 soft cap: c * tanh(out / c), c = epi_const;
  *                3 row gate: out *= sigmoid(epi_ptr[m * epi_row_stride + b]);
+ *                4 element-wise function chosen by act: 0 SiLU, 1 tanh-form GELU, 2 xIELU (a z^2 + z/2 for z > 0,
+ *                b (exp(z) - 1 - z) + z/2 otherwise, with a = epi_ptr[0], b = epi_ptr[1]), 3 out *= epi_const;
  *   out_dtype    NV_BF16 or NV_F32, independent of the operands' dtype. */
 int nv_linear(const void* a, int64_t a_row_stride, const int32_t* a_rows, const void* w, int64_t w_row_stride,
               const void* bias, void* out, int64_t out_row_stride, int out_dtype, int64_t M, int N, int K, int batch,
@@ -395,6 +397,61 @@ int nv_moe_sort(const int32_t* idx, int64_t tokens, int experts, int top, int32_
 int nv_moe_combine(const float* y, const int32_t* slot_of, const float* weights, int top, const float* shared,
                    const float* shared_gate, int64_t shared_gate_stride, float* out, int64_t tokens, int width,
                    nv_stream_t stream);
+
+/* ---- a residual kept as several fp32 streams, token shift (csrc/streams.hip) ----
+ * nv_embed_sinusoid: every stream of out[t] ([tokens, streams, width]) = table[ids[t]] + sinusoid(positions[t]) with
+ *   entry 2i = sin(p f_i), entry 2i+1 = cos(p f_i), f = inv_freq[i] (double, ceil(width / 2) entries).
+ * nv_hc_norm: with `delta` (the previous sublayer's output) the streams of a row are first replaced by
+ *   x'_t = sum_s mix[s][t] x_s + out[t] delta, mix/out from hc_prev = in[S] | out[S] | mix[S][S] (null: x_t + delta);
+ *   then u = sum_s hc_in[s] x_s (null: the plain sum) and out = u / sqrt(mean(u^2) + eps) * (w, or 1 + w with one_plus).
+ *   rows_idx gathers rows and leaves the streams as they are.  out is fp32 or the model's type.
+ * nv_token_shift: out[t] = h[t] + (h[t-1] - h[t]) * mu; the row before a portion comes from the request's slot of
+ *   state [slots, width] (zeros when past_lens is 0), which then receives the portion's last row.
+ * nv_group_rmsnorm_f32: fp32 rows of `groups` parts of n numbers, each part divided by its own root mean square. */
+int nv_embed_sinusoid(const int64_t* ids, const int64_t* positions, const void* table, const double* inv_freq, float* out,
+                      int64_t tokens, int streams, int width, int64_t vocab, int dtype, nv_stream_t stream);
+int nv_hc_norm(float* x, int streams, int width, const float* delta, int64_t delta_row_stride, const float* hc_prev,
+               const float* hc_in, const void* w, int one_plus, float eps, const int32_t* rows_idx, void* out,
+               int64_t out_row_stride, int out_dtype, int64_t rows, int dtype, nv_stream_t stream);
+int nv_token_shift(const float* h, const void* mu, float* state, const int32_t* cu_q, const int32_t* past_lens,
+                   const int32_t* state_slots, const int32_t* seq_of_token, void* out, int64_t tokens, int width,
+                   int dtype, nv_stream_t stream);
+int nv_group_rmsnorm_f32(const float* x, int64_t x_row_stride, const void* w, void* out, int64_t out_row_stride,
+                         int64_t rows, int groups, int n, float eps, int dtype, nv_stream_t stream);
+
+/* ---- softmax attention with shaped scores over a paged cache of rows [k: G * dim | v: G * vdim] (csrc/window_attn.hip) ----
+ * nv_qk_norm_store: per-head RMS norm of the fp32 q and k projections (weights shared by the heads), q * scale *
+ *   temp[h] left in fp32 [tokens, heads * dim], normalised k and v written to cache row slot_mapping[t] (-1: skipped).
+ * nv_window_attn: score = cap(q . k) - 2^(-8 (h + 1) / heads) * (i - j) over keys 0 <= i - j < window (0: all earlier),
+ *   cap(z) = softcap * tanh(z / softcap) (softcap 0: none); out[t][h * vdim ..] = out_scale * softmax-weighted values. */
+int nv_qk_norm_store(const float* proj, int64_t proj_row_stride, int q_off, int k_off, int v_off, const void* q_norm,
+                     const void* k_norm, const void* temp, float scale, float eps, const int32_t* slot_mapping,
+                     void* cache, float* q_out, int64_t tokens, int heads, int kv_heads, int dim, int vdim, int dtype,
+                     nv_stream_t stream);
+int nv_window_attn(const float* q, const void* cache, const int32_t* block_tables, int table_cols, const int32_t* cu_q,
+                   const int32_t* past_lens, const int32_t* seq_of_token, void* out, int64_t out_row_stride,
+                   int64_t tokens, int max_q, int heads, int kv_heads, int dim, int vdim, int block_size, int window,
+                   float softcap, float out_scale, int dtype, nv_stream_t stream);
+
+/* ---- recurrences with an fp32 state per request (csrc/scan.hip) ----
+ * nv_causal_conv: per-channel causal convolution over fp32 rows; state [slots, taps - 1, channels] keeps the last
+ *   inputs; act 0 none, 1 SiLU; results as fp32 rows and/or rows of the storage type.
+ * nv_rglru_scan: a = exp(-c sigmoid(gr) softplus(lam)), S = a S + sqrt(1 - a^2) sigmoid(gi) u, out = out_scale * S *
+ *   gelu_tanh(y); gates hold, per block of block_width channels, the gr logits followed by the gi logits.
+ * nv_ssd_scan: per head, S [state, vdim] <- exp(-exp(A_log) dt) S + dt B x^T, y = S^T C + D x, dt = softplus(raw +
+ *   dt_bias), out = y * silu(z) in fp32; xbc rows hold x | B | C with B and C shared by heads / groups heads. */
+int nv_causal_conv(const float* x, int64_t x_row_stride, const void* w, const void* bias, float* state,
+                   const int32_t* cu_q, const int32_t* past_lens, const int32_t* state_slots, const int32_t* seq_of_token,
+                   float* out_f32, int64_t out_f32_row_stride, void* out_t, int64_t out_t_row_stride, int64_t tokens,
+                   int channels, int taps, int act, int dtype, nv_stream_t stream);
+int nv_rglru_scan(const float* u, int64_t u_row_stride, const float* gates, int64_t gates_row_stride, const float* y,
+                  int64_t y_row_stride, const void* lam, float* state, const int32_t* cu_q, const int32_t* past_lens,
+                  const int32_t* state_slots, void* out, int64_t out_row_stride, int num_seqs, int channels,
+                  int block_width, float c, float out_scale, int dtype, nv_stream_t stream);
+int nv_ssd_scan(const float* xbc, int64_t xbc_row_stride, const float* z, int64_t z_row_stride, const float* dt,
+                int64_t dt_row_stride, const void* dt_bias, const void* A_log, const void* D, float* state,
+                const int32_t* cu_q, const int32_t* past_lens, const int32_t* state_slots, float* out, int num_seqs,
+                int heads, int groups, int state_size, int vdim, int dtype, nv_stream_t stream);
 
 #ifdef __cplusplus
 }
