@@ -217,7 +217,7 @@ extern "C" int nv_causal_conv(const float* x, int64_t x_row_stride, const void* 
                               const int32_t* seq_of_token, float* out_f32, int64_t out_f32_row_stride, void* out_t,
                               int64_t out_t_row_stride, int64_t tokens, int channels, int taps, int act, int dtype,
                               nv_stream_t stream) {
-  NV_CHECK_ARG(x && w && state && cu_q && past_lens && state_slots && seq_of_token && (out_f32 || out_t),
+  NV_CHECK_ARG(x && w && (state || taps == 1) && cu_q && past_lens && state_slots && seq_of_token && (out_f32 || out_t),
                "nv_causal_conv: null pointer");
   NV_CHECK_ARG(dtype == NV_BF16 || dtype == NV_F32, "nv_causal_conv: bad dtype %d", dtype);
   NV_CHECK_ARG(tokens >= 0 && tokens < (1ll << 31) && channels > 0 && taps >= 1 && taps <= CONV_MAX_TAPS &&
