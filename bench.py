@@ -282,7 +282,7 @@ def run_generate_workload(args):
     print(json.dumps(line), flush=True)
 
 
-# --arch-compare: the Rurutar design beside the closest model family the engine has (the dense Qwen3 decoder) at equal
+# --arch-compare: the Rurutar and Nonetar designs beside the dense Qwen3 decoder (and beside each other) at equal
 # width, depth, active feed-forward size and vocabulary, both through LLM.generate: prefill and decode tokens/s.
 # name: (width, layers, prompts, prompt length, decoded tokens)
 ARCH_COMPARE_SIZES = {
@@ -322,12 +322,38 @@ def rurutar_bench_config(width: int, layers: int, vocab: int = 32000):
     return rurutar_config(raw, None, dtype=torch.bfloat16)
 
 
+def nonetar_bench_config(width: int, layers: int, vocab: int = 32000):
+    """A Nonetar configuration with the proportions of a real model's layers: three of four layers run window attention
+    (two query heads per key head, 128-wide heads, window 512) beside a gated linear recurrence as wide as the model,
+    every fourth layer is a state-space mixer with twice the model's width inside (64-wide heads, 128 states); two
+    residual streams; feed-forwards of two matrices with the parameter count of the dense comparator's three."""
+    from byox_vllm_amd.models.nonetar import nonetar_config
+    heads = width // 128
+    par = {"type": "parallel",
+           "mixer": {"left": {"heads": heads, "kv_heads": max(1, heads // 2), "dim": 128, "vdim": 128, "mask": {"size": 512},
+                              "scale": 128 ** -0.5, "softcap": 50.0},
+                     "left_scale": 0.8, "right": {"width": width, "blocks": heads, "conv": 4}, "right_scale": 1.1}}
+    ssm = {"type": "mamba2", "mixer": {"heads": 2 * width // 64, "groups": 1, "vdim": 64, "state": 128, "conv": 4,
+                                       "norm_groups": 1}}
+    specs = []
+    for i in range(layers):
+        layer = json.loads(json.dumps(ssm if i % 4 == 3 else par))
+        layer["mlp"] = {"kind": "dense", "ff": 9 * width // 2}
+        specs.append(layer)
+    raw = {"architecture": "Nonetar", "vocab": vocab, "width": width, "streams": 2, "norm": {"eps": 1e-6},
+           "logit_scale": 0.25, "layers": specs}
+    return nonetar_config(raw, dtype=torch.bfloat16)
+
+
 def run_arch_compare(args):
     from byox_vllm_amd import LLM, SamplingParams
     from byox_vllm_amd.config import qwen2_config
     assert args.gpus == 1, "--arch-compare runs on one GPU"
     random.seed(0)
     results = []
+    designs = {"rurutar": rurutar_bench_config, "nonetar": nonetar_bench_config}
+    chosen = [d for d in args.arch_designs.split(",") if d]
+    assert chosen and all(d in designs for d in chosen), f"--arch-designs: a subset of {sorted(designs)}"
     for name, (width, layers, num, plen, decoded) in ARCH_COMPARE_SIZES.items():
         if args.arch_sizes and name not in args.arch_sizes.split(","):
             continue
@@ -337,7 +363,7 @@ def run_arch_compare(args):
                              num_hidden_layers=layers, num_attention_heads=width // 128, num_key_value_heads=width // 256,
                              head_dim=128, vocab_size=32000, tie_word_embeddings=False)
         row = {"size": name, "width": width, "layers": layers, "prompts": num, "prompt_len": plen, "decoded": decoded}
-        for label, hf in (("rurutar", rurutar_bench_config(width, layers)), ("qwen3_dense", dense)):
+        for label, hf in [(d, designs[d](width, layers)) for d in chosen] + [("qwen3_dense", dense)]:
             llm = LLM("synthetic", hf_config=hf, enforce_eager=args.eager, max_model_len=plen + decoded + 8,
                       max_num_seqs=num, max_num_batched_tokens=num * plen, kvcache_block_size=256,
                       num_kvcache_blocks=blocks)
@@ -358,7 +384,8 @@ def run_arch_compare(args):
                           "decode_tok_s": round(agg["decode_tokens"] / agg["decode_s"], 1),
                           "decode_ms_per_step": round(1e3 * agg["decode_s"] / agg["decode_steps"], 3)}
         results.append(row)
-    print(json.dumps({"metric": "prefill and decode tokens/s, Rurutar beside the dense Qwen3 decoder at equal size",
+    print(json.dumps({"metric": "prefill and decode tokens/s, " + " and ".join(d.capitalize() for d in chosen)
+                                + " beside the dense Qwen3 decoder at equal size",
                       "unit": "tokens/s", "n_gpus": 1, "dtype": "bf16", "data": "synthetic (random weights, random prompts)",
                       "higher_is_better": True, "sizes": results}), flush=True)
 
@@ -446,8 +473,10 @@ def main():
     ap.add_argument("--eager", action="store_true", help="no hipGraph (debug)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--arch-compare", action="store_true",
-                    help="instead of the decode benchmark: prefill and decode tokens/s of the Rurutar design beside the "
-                         "dense Qwen3 decoder at equal size (one GPU, LLM.generate)")
+                    help="instead of the decode benchmark: prefill and decode tokens/s of the designs named by --arch-designs "
+                         "beside the dense Qwen3 decoder at equal size (one GPU, LLM.generate)")
+    ap.add_argument("--arch-designs", default="rurutar",
+                    help="--arch-compare: the designs to run beside the dense decoder, comma-separated (rurutar, nonetar)")
     ap.add_argument("--arch-sizes", default="", help="--arch-compare: comma-separated subset of " + ",".join(ARCH_COMPARE_SIZES))
     args = ap.parse_args()
     if args.arch_compare:

@@ -107,26 +107,57 @@ struct RglruArgs {
   float c, out_scale;
 };
 
+// The recurrence S_t = a_t S_(t-1) + b_t is a composition of affine maps, so a request's tokens are cut into RG_CHUNKS
+// runs that are walked side by side: thread (channel, run) first folds its run into one map (A, B), the maps of the
+// earlier runs applied to the slot's value give the run's incoming state, and a second walk writes the outputs.
+// A step of one token per request costs one run's walk; a prompt's walk is RG_CHUNKS times shorter than the prompt.
+constexpr int RG_CHUNKS = 16, RG_CH = 64;
+
 template <typename T>
-__global__ __launch_bounds__(256) void rglru_scan_kernel(RglruArgs p) {
-  const int ch = blockIdx.x * blockDim.x + threadIdx.x;
+__global__ __launch_bounds__(RG_CHUNKS * RG_CH) void rglru_scan_kernel(RglruArgs p) {
+  __shared__ float sA[RG_CHUNKS][RG_CH], sB[RG_CHUNKS][RG_CH];
+  const int cx = threadIdx.x, j = threadIdx.y;
+  const int ch = blockIdx.x * RG_CH + cx;
   const int b = blockIdx.y;
-  if (ch >= p.C) return;
   const int t0 = p.cu_q[b], t1 = p.cu_q[b + 1];
   if (t1 <= t0) return;
-  float* slot = p.state + (int64_t)p.slots[b] * p.C + ch;
-  float S = p.past[b] == 0 ? 0.0f : *slot;
-  const float sp = p.c * softplus_f32(ld_f32<T>(reinterpret_cast<const T*>(p.lam) + ch));
-  const int gcol = (ch / p.bw) * 2 * p.bw + ch % p.bw;
-  T* out = reinterpret_cast<T*>(p.out);
-  for (int64_t t = t0; t < t1; ++t) {
+  const bool on = ch < p.C;
+  const int len = (t1 - t0 + RG_CHUNKS - 1) / RG_CHUNKS;
+  const int64_t c0 = min((int64_t)t1, (int64_t)t0 + (int64_t)j * len), c1 = min((int64_t)t1, c0 + len);
+  const float sp = on ? p.c * softplus_f32(ld_f32<T>(reinterpret_cast<const T*>(p.lam) + ch)) : 0.0f;
+  const int gcol = on ? (ch / p.bw) * 2 * p.bw + ch % p.bw : 0;
+  auto step = [&](int64_t t, float& a, float& inp) {
     const float gr = p.gates[t * p.g_rs + gcol], gi = p.gates[t * p.g_rs + gcol + p.bw];
     const float log_a = -sp * sigmoid_f32(gr);
+    a = expf(log_a);
     // sqrt(1 - a^2) through expm1: 1 - exp(2 log a) loses its digits when the decay is close to one
-    S = expf(log_a) * S + sqrtf(-expm1f(2.0f * log_a)) * sigmoid_f32(gi) * p.u[t * p.u_rs + ch];
+    inp = sqrtf(-expm1f(2.0f * log_a)) * sigmoid_f32(gi) * p.u[t * p.u_rs + ch];
+  };
+  float A = 1.0f, B = 0.0f;
+  if (on && t1 - t0 > 1) {
+    for (int64_t t = c0; t < c1; ++t) {
+      float a, inp;
+      step(t, a, inp);
+      A *= a;
+      B = a * B + inp;
+    }
+  }
+  sA[j][cx] = A;
+  sB[j][cx] = B;
+  __syncthreads();
+  if (!on) return;
+  float* slot = p.state + (int64_t)p.slots[b] * p.C + ch;
+  float S = p.past[b] == 0 ? 0.0f : *slot;
+  if (t1 - t0 > 1)
+    for (int jj = 0; jj < j; ++jj) S = sA[jj][cx] * S + sB[jj][cx];
+  T* out = reinterpret_cast<T*>(p.out);
+  for (int64_t t = c0; t < c1; ++t) {
+    float a, inp;
+    step(t, a, inp);
+    S = a * S + inp;
     st_f32<T>(out + t * p.out_rs + ch, S * gelu_tanh_f32(p.y[t * p.y_rs + ch]) * p.out_scale);
   }
-  *slot = S;
+  if (c1 == t1 && c1 > c0) *slot = S;      // the run that holds the step's last token
 }
 
 struct SsdArgs {
@@ -147,65 +178,84 @@ struct SsdArgs {
   int H, G, N, P, parts;
 };
 
-// One workgroup per (request, head); thread (part, v) keeps S[part + parts * i][v], i < DPT, in registers.
+// One workgroup per (request, head); thread (part, v) keeps S[part + parts * i][v], i < DPT, in registers.  Tokens are
+// staged `tc` at a time: step sizes and decays first, then dt * B, C and x rows in LDS; the walk over the staged tokens
+// needs no barrier (each thread leaves its partial y per token in LDS), the partial sums meet once per stage.
 template <typename T, int DPT>
-__global__ __launch_bounds__(1024) void ssd_scan_kernel(SsdArgs p) {
+__global__ __launch_bounds__(1024) void ssd_scan_kernel(SsdArgs p, int tc) {
   extern __shared__ float lds[];
-  float* sB = lds;                    // [N] dt * B
-  float* sC = sB + p.N;               // [N]
-  float* so = sC + p.N;               // [parts][P]
+  const int N = p.N, P = p.P, parts = p.parts;
+  float* sB = lds;                       // [tc][N] dt * B
+  float* sC = sB + tc * N;               // [tc][N]
+  float* sx = sC + tc * N;               // [tc][P]
+  float* so = sx + tc * P;               // [tc][parts][P]
+  float* sdt = so + tc * parts * P;      // [tc]
+  float* sdec = sdt + tc;                // [tc]
   const int h = blockIdx.x, b = blockIdx.y;
-  const int tid = threadIdx.x;
-  const bool active = tid < p.parts * p.P;
-  const int v = tid % p.P, part = tid / p.P;
+  const int tid = threadIdx.x, bd = blockDim.x;
+  const bool active = tid < parts * P;
+  const int v = tid % P, part = tid / P;
   const int t0 = p.cu_q[b], t1 = p.cu_q[b + 1];
   if (t1 <= t0) return;
   const int grp = h / (p.H / p.G);
-  float* S_g = p.state + ((int64_t)p.slots[b] * p.H + h) * p.N * p.P;
+  float* S_g = p.state + ((int64_t)p.slots[b] * p.H + h) * N * P;
   const bool fresh = p.past[b] == 0;
   float S[DPT];
 #pragma unroll
   for (int i = 0; i < DPT; ++i) {
-    const int n = part + p.parts * i;
-    S[i] = (active && n < p.N && !fresh) ? S_g[(int64_t)n * p.P + v] : 0.0f;
+    const int n = part + parts * i;
+    S[i] = (active && n < N && !fresh) ? S_g[(int64_t)n * P + v] : 0.0f;
   }
   const float rate = expf(ld_f32<T>(reinterpret_cast<const T*>(p.A_log) + h));
   const float dtb = ld_f32<T>(reinterpret_cast<const T*>(p.dt_bias) + h);
   const float Dh = ld_f32<T>(reinterpret_cast<const T*>(p.D) + h);
-  const int inner = p.H * p.P;
-  for (int64_t t = t0; t < t1; ++t) {
-    const float* row = p.xbc + t * p.xbc_rs;
-    const float dt = softplus_f32(p.dt[t * p.dt_rs + h] + dtb);
-    const float decay = expf(-rate * dt);
-    for (int j = tid; j < p.N; j += blockDim.x) {
-      sB[j] = dt * row[inner + grp * p.N + j];
-      sC[j] = row[inner + p.G * p.N + grp * p.N + j];
+  const int inner = p.H * P;
+  for (int64_t c0 = t0; c0 < t1; c0 += tc) {
+    const int nt = (int)min((int64_t)tc, t1 - c0);
+    if (tid < nt) {
+      const float dt = softplus_f32(p.dt[(c0 + tid) * p.dt_rs + h] + dtb);
+      sdt[tid] = dt;
+      sdec[tid] = expf(-rate * dt);
     }
-    const float xv = active ? row[h * p.P + v] : 0.0f;
     __syncthreads();
-    float o = 0.0f;
+    for (int i = tid; i < nt * N; i += bd) {
+      const int tt = i / N, n = i % N;
+      const float* row = p.xbc + (c0 + tt) * p.xbc_rs;
+      sB[i] = sdt[tt] * row[inner + grp * N + n];
+      sC[i] = row[inner + p.G * N + grp * N + n];
+    }
+    for (int i = tid; i < nt * P; i += bd) sx[i] = p.xbc[(c0 + i / P) * p.xbc_rs + h * P + i % P];
+    __syncthreads();
+    if (active) {
+      for (int tt = 0; tt < nt; ++tt) {
+        const float xv = sx[tt * P + v], decay = sdec[tt];
+        const float* Bt = sB + tt * N;
+        const float* Ct = sC + tt * N;
+        float o = 0.0f;
 #pragma unroll
-    for (int i = 0; i < DPT; ++i) {
-      const int n = part + p.parts * i;
-      if (n < p.N) {
-        S[i] = decay * S[i] + sB[n] * xv;
-        o += S[i] * sC[n];
+        for (int i = 0; i < DPT; ++i) {
+          const int n = part + parts * i;
+          if (n < N) {
+            S[i] = decay * S[i] + Bt[n] * xv;
+            o += S[i] * Ct[n];
+          }
+        }
+        so[(tt * parts + part) * P + v] = o;
       }
     }
-    if (active) so[part * p.P + v] = o;
     __syncthreads();
-    if (tid < p.P) {
-      float y = 0.0f;
-      for (int q = 0; q < p.parts; ++q) y += so[q * p.P + tid];
-      y += Dh * row[h * p.P + tid];
-      p.out[t * inner + h * p.P + tid] = y * silu_f32(p.z[t * p.z_rs + h * p.P + tid]);
+    for (int i = tid; i < nt * P; i += bd) {
+      const int tt = i / P, e = i % P;
+      float y = Dh * sx[i];
+      for (int q = 0; q < parts; ++q) y += so[(tt * parts + q) * P + e];
+      p.out[(c0 + tt) * inner + h * P + e] = y * silu_f32(p.z[(c0 + tt) * p.z_rs + h * P + e]);
     }
   }
   if (active) {
 #pragma unroll
     for (int i = 0; i < DPT; ++i) {
-      const int n = part + p.parts * i;
-      if (n < p.N) S_g[(int64_t)n * p.P + v] = S[i];
+      const int n = part + parts * i;
+      if (n < N) S_g[(int64_t)n * P + v] = S[i];
     }
   }
 }
@@ -244,9 +294,8 @@ extern "C" int nv_rglru_scan(const float* u, int64_t u_row_stride, const float* 
   if (num_seqs == 0) return NV_OK;
   RglruArgs p{u, u_row_stride, gates, gates_row_stride, y, y_row_stride, lam, state, cu_q, past_lens, state_slots, out,
               out_row_stride, channels, block_width, c, out_scale};
-  const int threads = 64;
-  NV_DISPATCH_T(dtype, rglru_scan_kernel<T><<<dim3((unsigned)((channels + threads - 1) / threads), (unsigned)num_seqs),
-                                              dim3(threads), 0, (hipStream_t)stream>>>(p));
+  NV_DISPATCH_T(dtype, rglru_scan_kernel<T><<<dim3((unsigned)((channels + RG_CH - 1) / RG_CH), (unsigned)num_seqs),
+                                              dim3(RG_CH, RG_CHUNKS), 0, (hipStream_t)stream>>>(p));
   NV_CHECK_LAUNCH();
   return NV_OK;
 }
@@ -271,12 +320,17 @@ extern "C" int nv_ssd_scan(const float* xbc, int64_t xbc_row_stride, const float
   SsdArgs p{xbc, xbc_row_stride, z, z_row_stride, dt, dt_row_stride, dt_bias, A_log, D, state, cu_q, past_lens,
             state_slots, out, heads, groups, state_size, vdim, parts};
   const int threads = ((parts * vdim + 63) / 64) * 64;
-  const size_t lds = (size_t)(2 * state_size + parts * vdim) * sizeof(float);
+  // tokens per stage: as many as fit 48 KB of LDS, at most 16
+  auto need = [&](int tc) { return (size_t)tc * (2 * state_size + vdim + parts * vdim + 2) * sizeof(float); };
+  int tc = 16;
+  while (tc > 1 && need(tc) > 48 * 1024) tc /= 2;
+  NV_CHECK_ARG(need(tc) <= 64 * 1024, "nv_ssd_scan: a token of %d + %d numbers does not fit the LDS", state_size, vdim);
+  const size_t lds = need(tc);
   dim3 grid((unsigned)heads, (unsigned)num_seqs);
   hipStream_t s = (hipStream_t)stream;
-  if (per <= 4) NV_DISPATCH_T(dtype, ssd_scan_kernel<T, 4><<<grid, dim3(threads), lds, s>>>(p));
-  else if (per <= 16) NV_DISPATCH_T(dtype, ssd_scan_kernel<T, 16><<<grid, dim3(threads), lds, s>>>(p));
-  else NV_DISPATCH_T(dtype, ssd_scan_kernel<T, 64><<<grid, dim3(threads), lds, s>>>(p));
+  if (per <= 4) NV_DISPATCH_T(dtype, ssd_scan_kernel<T, 4><<<grid, dim3(threads), lds, s>>>(p, tc));
+  else if (per <= 16) NV_DISPATCH_T(dtype, ssd_scan_kernel<T, 16><<<grid, dim3(threads), lds, s>>>(p, tc));
+  else NV_DISPATCH_T(dtype, ssd_scan_kernel<T, 64><<<grid, dim3(threads), lds, s>>>(p, tc));
   NV_CHECK_LAUNCH();
   return NV_OK;
 }

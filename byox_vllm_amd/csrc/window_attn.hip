@@ -178,6 +178,197 @@ __global__ __launch_bounds__(256) void window_attn_kernel(WAttnArgs p) {
   }
 }
 
+// ---- the same attention on the matrix cores (bf16 cache) ----
+// A workgroup of four wavefronts owns up to 64 query rows, 16 per wavefront: TQ consecutive tokens times the R heads
+// that share key/value head g.  Per tile of 64 keys the K rows are staged row-major and the V rows transposed (both
+// bf16, zero-filled past the last key); every wavefront computes S = Q K^T for its rows with the queries held as
+// register fragments, shapes and masks the scores in the accumulator layout (a lane owns four rows of one key column),
+// keeps running maxima and sums per row with 16-lane reductions, passes P through a private LDS patch to turn it into an
+// A operand, and accumulates O += P V.  Scores, maxima, sums and rescaling are fp32; Q and P enter the MFMAs as bf16.
+constexpr int MA_KEYS = 64, MA_VST = MA_KEYS + 8, MA_PST = MA_KEYS + 8;
+
+template <int KS, int CT>
+__global__ __launch_bounds__(256) void window_attn_mfma_kernel(WAttnArgs p) {
+  constexpr int DK = KS * 32, KST = DK + 8, DVP = CT * 16;
+  extern __shared__ u32x4 lds_raw[];
+  bf16_t* sK = reinterpret_cast<bf16_t*>(lds_raw);          // [64][KST]
+  bf16_t* sVt = sK + MA_KEYS * KST;                          // [DVP][MA_VST]
+  bf16_t* sP = sVt + DVP * MA_VST;                           // [4][16][MA_PST]
+  __shared__ int64_t sRow[MA_KEYS];
+  const int R = p.H / p.G, d = p.d, dv = p.dv;
+  const int g = blockIdx.y;
+  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  const int lc = lane & 15, lg = lane >> 4;
+  const int64_t t_begin = (int64_t)blockIdx.x * p.TQ;
+  const int64_t t_end = min(p.tokens, t_begin + p.TQ);
+  const bf16_t* cache = reinterpret_cast<const bf16_t*>(p.cache);
+  const int cw = p.G * (d + dv);
+  bf16_t* out = reinterpret_cast<bf16_t*>(p.out);
+  bf16_t* sPw = sP + wv * 16 * MA_PST;
+
+  for (int64_t ts = t_begin; ts < t_end;) {
+    const int b = p.seq_of[ts];
+    const int64_t te = min(t_end, (int64_t)p.cu_q[b + 1]);
+    const int nq = (int)(te - ts), rows = nq * R;
+    const int p0 = p.past[b] + (int)(ts - p.cu_q[b]);
+    const int32_t* table = p.tables + (int64_t)b * p.table_cols;
+    const bool wave_on = wv * 16 < rows;
+    // query fragments of this wavefront's 16 rows (A operand: lane holds row lc, features 8 lg .. 8 lg + 7 of each step)
+    bf16x8 qf[KS];
+    {
+      const int rr = wv * 16 + lc;
+      const bool ok = rr < rows;
+      const float* qrow = ok ? p.q + ((ts + rr / R) * p.H + g * R + rr % R) * d : nullptr;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const int e = ks * 32 + lg * 8 + i;
+          qf[ks][i] = (bf16_t)((ok && e < d) ? qrow[e] : 0.0f);
+        }
+      }
+    }
+    // the four accumulator rows of this lane
+    int pos[4];
+    float slope[4], m_run[4], l_run[4];
+    bool valid[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int rr = wv * 16 + lg * 4 + r;
+      valid[r] = rr < rows;
+      pos[r] = p0 + rr / R;
+      slope[r] = exp2f(-8.0f * (float)(g * R + rr % R + 1) / (float)p.H);
+      m_run[r] = -INFINITY;
+      l_run[r] = 0.0f;
+    }
+    f32x4 acc_o[CT];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) acc_o[ct] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    const int wpos_lo = p0 + (wv * 16) / R, wpos_hi = p0 + min(rows - 1, wv * 16 + 15) / R;
+
+    const int lo = p.window > 0 ? max(0, p0 - p.window + 1) : 0, hi = p0 + nq - 1;
+    for (int j0 = lo; j0 <= hi; j0 += MA_KEYS) {
+      if (tid < MA_KEYS) {
+        const int kp = j0 + tid;
+        sRow[tid] = kp <= hi ? (int64_t)table[kp / p.block_size] * p.block_size + kp % p.block_size : -1;
+      }
+      __syncthreads();
+      for (int c = tid; c < MA_KEYS * (DK / 8); c += 256) {
+        const int key = c / (DK / 8), part = c % (DK / 8);
+        const int64_t row = sRow[key];
+        u32x4 val = u32x4{0u, 0u, 0u, 0u};
+        if (row >= 0 && part * 8 < d) val = *reinterpret_cast<const u32x4*>(cache + row * cw + g * d + part * 8);
+        *reinterpret_cast<u32x4*>(sK + key * KST + part * 8) = val;
+      }
+      for (int c = tid; c < MA_KEYS * (DVP / 8); c += 256) {
+        const int key = c % MA_KEYS, part = c / MA_KEYS;
+        const int64_t row = sRow[key];
+        u32x4 val = u32x4{0u, 0u, 0u, 0u};
+        if (row >= 0 && part * 8 < dv) val = *reinterpret_cast<const u32x4*>(cache + row * cw + p.G * d + g * dv + part * 8);
+        uint16_t* dst = reinterpret_cast<uint16_t*>(sVt) + (part * 8) * MA_VST + key;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          dst[(2 * i) * MA_VST] = (uint16_t)(val[i] & 0xffffu);
+          dst[(2 * i + 1) * MA_VST] = (uint16_t)(val[i] >> 16);
+        }
+      }
+      __syncthreads();
+      // keys this wavefront's rows can see: [wpos_lo - window + 1, wpos_hi]
+      const bool need = wave_on && j0 <= wpos_hi && (p.window <= 0 || j0 + MA_KEYS - 1 > wpos_lo - p.window);
+      if (need) {
+        f32x4 acc_s[4];
+#pragma unroll
+        for (int sub = 0; sub < 4; ++sub) {
+          acc_s[sub] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+          for (int ks = 0; ks < KS; ++ks) {
+            const bf16x8 kf = *reinterpret_cast<const bf16x8*>(sK + (sub * 16 + lc) * KST + ks * 32 + lg * 8);
+            acc_s[sub] = mfma16(qf[ks], kf, acc_s[sub]);
+          }
+        }
+        float corr[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          float mt = -INFINITY;
+#pragma unroll
+          for (int sub = 0; sub < 4; ++sub) {
+            const int kp = j0 + sub * 16 + lc;
+            const int dist = pos[r] - kp;
+            float sc = acc_s[sub][r];
+            if (p.softcap > 0.0f) sc = p.softcap * tanhf(sc / p.softcap);
+            sc -= slope[r] * (float)dist;
+            const bool vis = valid[r] && dist >= 0 && (p.window <= 0 || dist < p.window);
+            sc = vis ? sc : -INFINITY;
+            acc_s[sub][r] = sc;
+            mt = fmaxf(mt, sc);
+          }
+#pragma unroll
+          for (int o = 1; o < 16; o <<= 1) mt = fmaxf(mt, __shfl_xor(mt, o, 64));
+          const float m_new = fmaxf(m_run[r], mt);
+          corr[r] = m_new == -INFINITY ? 1.0f : __expf(m_run[r] - m_new);
+          float sum = 0.0f;
+#pragma unroll
+          for (int sub = 0; sub < 4; ++sub) {
+            const float sc = acc_s[sub][r];
+            const float e = sc == -INFINITY ? 0.0f : __expf(sc - m_new);
+            sum += e;
+            sPw[(lg * 4 + r) * MA_PST + sub * 16 + lc] = (bf16_t)e;
+          }
+#pragma unroll
+          for (int o = 1; o < 16; o <<= 1) sum += __shfl_xor(sum, o, 64);
+          l_run[r] = l_run[r] * corr[r] + sum;
+          m_run[r] = m_new;
+        }
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) acc_o[ct][r] *= corr[r];
+        // the patch is private to this wavefront: its own LDS accesses complete in order
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int ks = 0; ks < MA_KEYS / 32; ++ks) {
+          const bf16x8 pf = *reinterpret_cast<const bf16x8*>(sPw + lc * MA_PST + ks * 32 + lg * 8);
+#pragma unroll
+          for (int ct = 0; ct < CT; ++ct) {
+            const bf16x8 vf = *reinterpret_cast<const bf16x8*>(sVt + (ct * 16 + lc) * MA_VST + ks * 32 + lg * 8);
+            acc_o[ct] = mfma16(pf, vf, acc_o[ct]);
+          }
+        }
+      }
+      __syncthreads();
+    }
+    if (wave_on) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int rr = wv * 16 + lg * 4 + r;
+        if (!valid[r]) continue;
+        const float f = p.out_scale / l_run[r];
+        bf16_t* orow = out + (ts + rr / R) * p.out_rs + (g * R + rr % R) * dv;
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) {
+          const int e = ct * 16 + lc;
+          if (e < dv) orow[e] = (bf16_t)(acc_o[ct][r] * f);
+        }
+      }
+    }
+    ts = te;
+  }
+}
+
+template <int KS>
+hipError_t launch_window_mfma(const WAttnArgs& p, int ct, dim3 grid, hipStream_t s) {
+  const size_t lds = ((size_t)MA_KEYS * (KS * 32 + 8) + (size_t)ct * 16 * MA_VST + 4 * 16 * MA_PST) * sizeof(bf16_t);
+  switch (ct) {
+    case 2: window_attn_mfma_kernel<KS, 2><<<grid, dim3(256), lds, s>>>(p); break;
+    case 4: window_attn_mfma_kernel<KS, 4><<<grid, dim3(256), lds, s>>>(p); break;
+    case 8: window_attn_mfma_kernel<KS, 8><<<grid, dim3(256), lds, s>>>(p); break;
+    default: window_attn_mfma_kernel<KS, 16><<<grid, dim3(256), lds, s>>>(p); break;
+  }
+  return hipGetLastError();
+}
+
 }  // namespace
 
 extern "C" int nv_qk_norm_store(const float* proj, int64_t proj_row_stride, int q_off, int k_off, int v_off,
@@ -207,6 +398,27 @@ extern "C" int nv_window_attn(const float* q, const void* cache, const int32_t* 
                "nv_window_attn: bad shape");
   if (tokens == 0) return NV_OK;
   const int R = heads / kv_heads;
+  // bf16 caches with 16-byte-aligned heads of up to 256 numbers: the matrix-core kernel
+  if (dtype == NV_BF16 && dim % 8 == 0 && vdim % 8 == 0 && dim <= 256 && vdim <= 256 && R <= 64 && kv_heads <= 65535 &&
+      (uintptr_t)cache % 16 == 0 && getenv("NV_WINDOW_ATTN_MFMA_OFF") == nullptr) {
+    const int ks = dim <= 64 ? 2 : dim <= 128 ? 4 : 8;
+    const int ct = vdim <= 32 ? 2 : vdim <= 64 ? 4 : vdim <= 128 ? 8 : 16;
+    const size_t lds = ((size_t)MA_KEYS * (ks * 32 + 8) + (size_t)ct * 16 * MA_VST + 4 * 16 * MA_PST) * 2;
+    if (lds <= 64 * 1024) {
+      const int TQm = max_q <= 1 ? 1 : 64 / R;
+      WAttnArgs pm{q, cache, block_tables, table_cols, cu_q, past_lens, seq_of_token, out, out_row_stride, tokens, heads,
+                   kv_heads, dim, vdim, block_size, window, TQm, MA_KEYS, softcap, out_scale};
+      dim3 gridm((unsigned)((tokens + TQm - 1) / TQm), (unsigned)kv_heads);
+      hipStream_t st = (hipStream_t)stream;
+      const hipError_t e = ks == 2 ? launch_window_mfma<2>(pm, ct, gridm, st)
+                           : ks == 4 ? launch_window_mfma<4>(pm, ct, gridm, st) : launch_window_mfma<8>(pm, ct, gridm, st);
+      if (e != hipSuccess) {
+        nv_set_error("nv_window_attn: %s", hipGetErrorString(e));
+        return NV_ERR_LAUNCH;
+      }
+      return NV_OK;
+    }
+  }
   const size_t budget = 64 * 1024;
   auto need = [&](int tq, int tk) {
     const size_t rows = (size_t)tq * R;

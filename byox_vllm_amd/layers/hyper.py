@@ -31,6 +31,7 @@ class StreamNorm(nn.Module):
             init = torch.cat([torch.ones(2 * S, dtype=torch.float32), torch.eye(S, dtype=torch.float32).flatten()])
             self.hc = nn.Parameter(init, requires_grad=False)
             self.hc.weight_loader = self._load_hc
+            self.hc.keep_init = True              # random initialisation leaves the identity in place
         else:
             self.register_parameter("hc", None)
 

@@ -110,6 +110,8 @@ def init_random_weights(model: nn.Module, seed: int = 0) -> None:
         if name == "lm_head.weight" and hasattr(model, "model") and \
                 param.data_ptr() == model.model.embed_tokens.weight.data_ptr():
             continue
+        if getattr(param, "keep_init", False):       # constructed with its neutral value (identity connections)
+            continue
         if name.endswith((".b", ".bias")) and "norm" in name:
             param.data.zero_()
             continue
