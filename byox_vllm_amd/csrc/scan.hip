@@ -176,11 +176,21 @@ struct SsdArgs {
   const int32_t* slots;
   float* out;             // [tokens, H * P]
   int H, G, N, P, parts;
+  // long prompts: runs of run_len tokens are walked side by side (see ssd_scan_kernel)
+  float* ws_state;        // [B * H * runs][N * P] state at the end of each run
+  float* ws_decay;        // [B * H * runs] product of the run's decays
+  int runs, run_len, pass;
 };
 
-// One workgroup per (request, head); thread (part, v) keeps S[part + parts * i][v], i < DPT, in registers.  Tokens are
-// staged `tc` at a time: step sizes and decays first, then dt * B, C and x rows in LDS; the walk over the staged tokens
-// needs no barrier (each thread leaves its partial y per token in LDS), the partial sums meet once per stage.
+// One workgroup per (request, head, run); thread (part, v) keeps S[part + parts * i][v], i < DPT, in registers.  Tokens
+// are staged `tc` at a time: step sizes and decays first, then dt * B, C and x rows in LDS; the walk over the staged
+// tokens needs no barrier (each thread leaves its partial y per token in LDS), the partial sums meet once per stage.
+//
+// S_t = decay_t S_(t-1) + U_t is an affine map of the state with a scalar factor, so a long prompt is cut into runs
+// that are walked side by side.  Pass 1: run 0 starts from the request's slot and is final; every other run starts
+// from zero, writes nothing but its end state E_j and the product D_j of its decays.  Pass 2: run j >= 1 starts from
+// S = E_0, S <- D_i S + E_i for 0 < i < j, and walks again, now writing its outputs; the run that holds the step's last
+// token leaves the state in the slot (nobody reads the slot in pass 2).  runs == 1 is the plain walk.
 template <typename T, int DPT>
 __global__ __launch_bounds__(1024) void ssd_scan_kernel(SsdArgs p, int tc) {
   extern __shared__ float lds[];
@@ -192,26 +202,47 @@ __global__ __launch_bounds__(1024) void ssd_scan_kernel(SsdArgs p, int tc) {
   float* sdt = so + tc * parts * P;      // [tc]
   float* sdec = sdt + tc;                // [tc]
   const int h = blockIdx.x, b = blockIdx.y;
+  const int j = blockIdx.z + (p.pass == 2 ? 1 : 0);
   const int tid = threadIdx.x, bd = blockDim.x;
   const bool active = tid < parts * P;
   const int v = tid % P, part = tid / P;
   const int t0 = p.cu_q[b], t1 = p.cu_q[b + 1];
-  if (t1 <= t0) return;
+  const int64_t cb = p.runs > 1 ? (int64_t)t0 + (int64_t)j * p.run_len : t0;
+  const int64_t ce = p.runs > 1 ? min((int64_t)t1, cb + p.run_len) : t1;
+  if (cb >= ce) return;
+  const bool emit = p.pass == 2 || j == 0;
   const int grp = h / (p.H / p.G);
   float* S_g = p.state + ((int64_t)p.slots[b] * p.H + h) * N * P;
+  const int64_t wrow = ((int64_t)b * p.H + h) * p.runs;
   const bool fresh = p.past[b] == 0;
   float S[DPT];
 #pragma unroll
   for (int i = 0; i < DPT; ++i) {
-    const int n = part + parts * i;
-    S[i] = (active && n < N && !fresh) ? S_g[(int64_t)n * P + v] : 0.0f;
+    const int n = part * DPT + i;
+    const bool mine = active && n < N;
+    if (j == 0) S[i] = (mine && !fresh) ? S_g[(int64_t)n * P + v] : 0.0f;
+    else if (p.pass == 1) S[i] = 0.0f;
+    else S[i] = mine ? p.ws_state[wrow * N * P + (int64_t)n * P + v] : 0.0f;
+  }
+  if (p.pass == 2) {
+    for (int r = 1; r < j; ++r) {
+      const float Dr = p.ws_decay[wrow + r];
+      const float* E = p.ws_state + (wrow + r) * N * P;
+#pragma unroll
+      for (int i = 0; i < DPT; ++i) {
+        const int n = part * DPT + i;
+        if (active && n < N) S[i] = Dr * S[i] + E[(int64_t)n * P + v];
+      }
+    }
   }
   const float rate = expf(ld_f32<T>(reinterpret_cast<const T*>(p.A_log) + h));
   const float dtb = ld_f32<T>(reinterpret_cast<const T*>(p.dt_bias) + h);
   const float Dh = ld_f32<T>(reinterpret_cast<const T*>(p.D) + h);
   const int inner = p.H * P;
-  for (int64_t c0 = t0; c0 < t1; c0 += tc) {
-    const int nt = (int)min((int64_t)tc, t1 - c0);
+  const bool vec4 = N % 4 == 0;
+  float dt_sum = 0.0f;
+  for (int64_t c0 = cb; c0 < ce; c0 += tc) {
+    const int nt = (int)min((int64_t)tc, ce - c0);
     if (tid < nt) {
       const float dt = softplus_f32(p.dt[(c0 + tid) * p.dt_rs + h] + dtb);
       sdt[tid] = dt;
@@ -231,32 +262,57 @@ __global__ __launch_bounds__(1024) void ssd_scan_kernel(SsdArgs p, int tc) {
         const float xv = sx[tt * P + v], decay = sdec[tt];
         const float* Bt = sB + tt * N;
         const float* Ct = sC + tt * N;
+        dt_sum += sdt[tt];
         float o = 0.0f;
+        if (vec4) {           // four state rows per LDS read (the rows of a thread are consecutive)
 #pragma unroll
-        for (int i = 0; i < DPT; ++i) {
-          const int n = part + parts * i;
-          if (n < N) {
-            S[i] = decay * S[i] + Bt[n] * xv;
-            o += S[i] * Ct[n];
+          for (int i = 0; i < DPT; i += 4) {
+            const int n = part * DPT + i;
+            if (n < N) {
+              const f32x4 b4 = *reinterpret_cast<const f32x4*>(Bt + n), c4 = *reinterpret_cast<const f32x4*>(Ct + n);
+#pragma unroll
+              for (int e = 0; e < 4; ++e) {
+                S[i + e] = decay * S[i + e] + b4[e] * xv;
+                o += S[i + e] * c4[e];
+              }
+            }
+          }
+        } else {
+#pragma unroll
+          for (int i = 0; i < DPT; ++i) {
+            const int n = part * DPT + i;
+            if (n < N) {
+              S[i] = decay * S[i] + Bt[n] * xv;
+              o += S[i] * Ct[n];
+            }
           }
         }
         so[(tt * parts + part) * P + v] = o;
       }
     }
     __syncthreads();
-    for (int i = tid; i < nt * P; i += bd) {
-      const int tt = i / P, e = i % P;
-      float y = Dh * sx[i];
-      for (int q = 0; q < parts; ++q) y += so[(tt * parts + q) * P + e];
-      p.out[(c0 + tt) * inner + h * P + e] = y * silu_f32(p.z[(c0 + tt) * p.z_rs + h * P + e]);
+    if (emit) {
+      for (int i = tid; i < nt * P; i += bd) {
+        const int tt = i / P, e = i % P;
+        float y = Dh * sx[i];
+        for (int q = 0; q < parts; ++q) y += so[(tt * parts + q) * P + e];
+        p.out[(c0 + tt) * inner + h * P + e] = y * silu_f32(p.z[(c0 + tt) * p.z_rs + h * P + e]);
+      }
     }
   }
   if (active) {
+    const bool to_slot = emit && ce == t1;
+    const bool to_ws = p.runs > 1 && p.pass == 1;
+    float* E = p.ws_state + (wrow + j) * N * P;
 #pragma unroll
     for (int i = 0; i < DPT; ++i) {
-      const int n = part + parts * i;
-      if (n < N) S_g[(int64_t)n * P + v] = S[i];
+      const int n = part * DPT + i;
+      if (n < N) {
+        if (to_slot) S_g[(int64_t)n * P + v] = S[i];
+        if (to_ws) E[(int64_t)n * P + v] = S[i];
+      }
     }
+    if (to_ws && tid == 0) p.ws_decay[wrow + j] = expf(-rate * dt_sum);
   }
 }
 
@@ -300,10 +356,29 @@ extern "C" int nv_rglru_scan(const float* u, int64_t u_row_stride, const float* 
   return NV_OK;
 }
 
+// runs a request of max_q tokens is cut into, and their length.  Runs cost every token a second walk, so they pay only
+// while (requests x heads) leaves most of the chip idle.
+static void ssd_runs(int num_seqs, int heads, int max_q, int* runs, int* run_len) {
+  *runs = 1;
+  *run_len = max_q > 0 ? max_q : 1;
+  if (max_q < 256 || (int64_t)num_seqs * heads >= 128) return;
+  int len = 128;
+  if ((max_q + len - 1) / len > 64) len = ((max_q + 63) / 64 + 15) / 16 * 16;
+  *run_len = len;
+  *runs = (max_q + len - 1) / len;
+}
+
+extern "C" size_t nv_ssd_scan_workspace_bytes(int num_seqs, int heads, int state_size, int vdim, int max_q) {
+  int runs, len;
+  ssd_runs(num_seqs, heads, max_q, &runs, &len);
+  return runs > 1 ? (size_t)num_seqs * heads * runs * ((size_t)state_size * vdim + 1) * sizeof(float) : 0;
+}
+
 extern "C" int nv_ssd_scan(const float* xbc, int64_t xbc_row_stride, const float* z, int64_t z_row_stride, const float* dt,
                            int64_t dt_row_stride, const void* dt_bias, const void* A_log, const void* D, float* state,
                            const int32_t* cu_q, const int32_t* past_lens, const int32_t* state_slots, float* out,
-                           int num_seqs, int heads, int groups, int state_size, int vdim, int dtype, nv_stream_t stream) {
+                           int num_seqs, int heads, int groups, int state_size, int vdim, int max_q, void* workspace,
+                           size_t workspace_bytes, int dtype, nv_stream_t stream) {
   NV_CHECK_ARG(xbc && z && dt && dt_bias && A_log && D && state && cu_q && past_lens && state_slots && out,
                "nv_ssd_scan: null pointer");
   NV_CHECK_ARG(dtype == NV_BF16 || dtype == NV_F32, "nv_ssd_scan: bad dtype %d", dtype);
@@ -317,8 +392,16 @@ extern "C" int nv_ssd_scan(const float* xbc, int64_t xbc_row_stride, const float
   if (parts > 8) parts = 8;
   const int per = (state_size + parts - 1) / parts;
   NV_CHECK_ARG(per <= 64, "nv_ssd_scan: a state of %d x %d exceeds one workgroup's registers", state_size, vdim);
+  int runs, run_len;
+  ssd_runs(num_seqs, heads, max_q, &runs, &run_len);
+  if (runs > 1) {
+    NV_CHECK_ARG(workspace && workspace_bytes >= nv_ssd_scan_workspace_bytes(num_seqs, heads, state_size, vdim, max_q),
+                 "nv_ssd_scan: %d runs need a workspace of nv_ssd_scan_workspace_bytes", runs);
+  }
+  float* ws_state = reinterpret_cast<float*>(workspace);
+  float* ws_decay = runs > 1 ? ws_state + (size_t)num_seqs * heads * runs * state_size * vdim : nullptr;
   SsdArgs p{xbc, xbc_row_stride, z, z_row_stride, dt, dt_row_stride, dt_bias, A_log, D, state, cu_q, past_lens,
-            state_slots, out, heads, groups, state_size, vdim, parts};
+            state_slots, out, heads, groups, state_size, vdim, parts, ws_state, ws_decay, runs, run_len, 1};
   const int threads = ((parts * vdim + 63) / 64) * 64;
   // tokens per stage: as many as fit 48 KB of LDS, at most 16
   auto need = [&](int tc) { return (size_t)tc * (2 * state_size + vdim + parts * vdim + 2) * sizeof(float); };
@@ -326,11 +409,14 @@ extern "C" int nv_ssd_scan(const float* xbc, int64_t xbc_row_stride, const float
   while (tc > 1 && need(tc) > 48 * 1024) tc /= 2;
   NV_CHECK_ARG(need(tc) <= 64 * 1024, "nv_ssd_scan: a token of %d + %d numbers does not fit the LDS", state_size, vdim);
   const size_t lds = need(tc);
-  dim3 grid((unsigned)heads, (unsigned)num_seqs);
   hipStream_t s = (hipStream_t)stream;
-  if (per <= 4) NV_DISPATCH_T(dtype, ssd_scan_kernel<T, 4><<<grid, dim3(threads), lds, s>>>(p, tc));
-  else if (per <= 16) NV_DISPATCH_T(dtype, ssd_scan_kernel<T, 16><<<grid, dim3(threads), lds, s>>>(p, tc));
-  else NV_DISPATCH_T(dtype, ssd_scan_kernel<T, 64><<<grid, dim3(threads), lds, s>>>(p, tc));
-  NV_CHECK_LAUNCH();
+  for (int pass = 1; pass <= (runs > 1 ? 2 : 1); ++pass) {
+    p.pass = pass;
+    dim3 grid((unsigned)heads, (unsigned)num_seqs, (unsigned)(pass == 1 ? runs : runs - 1));
+    if (per <= 4) NV_DISPATCH_T(dtype, ssd_scan_kernel<T, 4><<<grid, dim3(threads), lds, s>>>(p, tc));
+    else if (per <= 16) NV_DISPATCH_T(dtype, ssd_scan_kernel<T, 16><<<grid, dim3(threads), lds, s>>>(p, tc));
+    else NV_DISPATCH_T(dtype, ssd_scan_kernel<T, 64><<<grid, dim3(threads), lds, s>>>(p, tc));
+    NV_CHECK_LAUNCH();
+  }
   return NV_OK;
 }

@@ -45,10 +45,15 @@ struct HcArgs {
   float eps;
 };
 
-template <typename T, typename TO>
+template <int V> struct VecOfFloats { typedef float type __attribute__((ext_vector_type(V))); };
+template <> struct VecOfFloats<1> { typedef float type; };
+
+// V numbers per thread and step: 4 (16-byte accesses to the streams) when the width and the strides allow it, else 1.
+template <typename T, typename TO, int V>
 __global__ __launch_bounds__(256) void hc_norm_kernel(HcArgs p) {
   extern __shared__ float su[];      // [W] the weighted sum of the streams
   __shared__ float red[32];
+  typedef typename VecOfFloats<V>::type vec;
   const int64_t i = blockIdx.x;
   const int64_t r = p.rows_idx ? p.rows_idx[i] : i;
   const int S = p.S, W = p.W;
@@ -56,16 +61,16 @@ __global__ __launch_bounds__(256) void hc_norm_kernel(HcArgs p) {
   const float* po = p.hc_prev ? p.hc_prev + S : nullptr;
   const float* pm = p.hc_prev ? p.hc_prev + 2 * S : nullptr;
   float ss = 0.0f;
-  for (int j = threadIdx.x; j < W; j += blockDim.x) {
-    float xs[HC_MAX_STREAMS];
+  for (int j = threadIdx.x * V; j < W; j += blockDim.x * V) {
+    vec xs[HC_MAX_STREAMS];
 #pragma unroll
-    for (int s = 0; s < HC_MAX_STREAMS; ++s) xs[s] = s < S ? xr[(int64_t)s * W + j] : 0.0f;
+    for (int s = 0; s < HC_MAX_STREAMS; ++s) xs[s] = s < S ? *reinterpret_cast<const vec*>(xr + (int64_t)s * W + j) : vec(0.0f);
     if (p.delta) {
-      const float y = p.delta[r * p.delta_rs + j];
-      float nx[HC_MAX_STREAMS];
+      const vec y = *reinterpret_cast<const vec*>(p.delta + r * p.delta_rs + j);
+      vec nx[HC_MAX_STREAMS];
 #pragma unroll
       for (int t = 0; t < HC_MAX_STREAMS; ++t) {
-        float v = 0.0f;
+        vec v = vec(0.0f);
         if (t < S) {
           if (pm) {
 #pragma unroll
@@ -75,19 +80,24 @@ __global__ __launch_bounds__(256) void hc_norm_kernel(HcArgs p) {
           } else {
             v = xs[t] + y;
           }
-          if (!p.rows_idx) xr[(int64_t)t * W + j] = v;
+          if (!p.rows_idx) *reinterpret_cast<vec*>(xr + (int64_t)t * W + j) = v;
         }
         nx[t] = v;
       }
 #pragma unroll
       for (int s = 0; s < HC_MAX_STREAMS; ++s) xs[s] = nx[s];
     }
-    float u = 0.0f;
+    vec u = vec(0.0f);
 #pragma unroll
     for (int s = 0; s < HC_MAX_STREAMS; ++s)
       if (s < S) u += p.hc_in ? p.hc_in[s] * xs[s] : xs[s];
-    su[j] = u;
-    ss += u * u;
+    *reinterpret_cast<vec*>(su + j) = u;
+    if constexpr (V == 1) {
+      ss += u * u;
+    } else {
+#pragma unroll
+      for (int e = 0; e < V; ++e) ss += u[e] * u[e];
+    }
   }
   ss = block_sum(ss, red);
   const float inv = 1.0f / sqrtf(ss / (float)W + p.eps);
@@ -173,9 +183,18 @@ extern "C" int nv_hc_norm(float* x, int streams, int width, const float* delta, 
   HcArgs p{x, delta, delta_row_stride, hc_prev, hc_in, w, rows_idx, out, out_row_stride, streams, width, one_plus, eps};
   const size_t lds = (size_t)width * sizeof(float);
   hipStream_t s = (hipStream_t)stream;
-  if (dtype == NV_F32) hc_norm_kernel<float, float><<<dim3((unsigned)rows), dim3(256), lds, s>>>(p);
-  else if (out_dtype == NV_F32) hc_norm_kernel<bf16_t, float><<<dim3((unsigned)rows), dim3(256), lds, s>>>(p);
-  else hc_norm_kernel<bf16_t, bf16_t><<<dim3((unsigned)rows), dim3(256), lds, s>>>(p);
+  const bool vec = width % 4 == 0 && (uintptr_t)x % 16 == 0 &&
+                   (!delta || ((uintptr_t)delta % 16 == 0 && delta_row_stride % 4 == 0));
+  const dim3 g((unsigned)rows), b(256);
+  if (vec) {
+    if (dtype == NV_F32) hc_norm_kernel<float, float, 4><<<g, b, lds, s>>>(p);
+    else if (out_dtype == NV_F32) hc_norm_kernel<bf16_t, float, 4><<<g, b, lds, s>>>(p);
+    else hc_norm_kernel<bf16_t, bf16_t, 4><<<g, b, lds, s>>>(p);
+  } else {
+    if (dtype == NV_F32) hc_norm_kernel<float, float, 1><<<g, b, lds, s>>>(p);
+    else if (out_dtype == NV_F32) hc_norm_kernel<bf16_t, float, 1><<<g, b, lds, s>>>(p);
+    else hc_norm_kernel<bf16_t, bf16_t, 1><<<g, b, lds, s>>>(p);
+  }
   NV_CHECK_LAUNCH();
   return NV_OK;
 }

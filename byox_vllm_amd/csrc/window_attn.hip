@@ -185,26 +185,52 @@ __global__ __launch_bounds__(256) void window_attn_kernel(WAttnArgs p) {
 // register fragments, shapes and masks the scores in the accumulator layout (a lane owns four rows of one key column),
 // keeps running maxima and sums per row with 16-lane reductions, passes P through a private LDS patch to turn it into an
 // A operand, and accumulates O += P V.  Scores, maxima, sums and rescaling are fp32; Q and P enter the MFMAs as bf16.
+//
+// SPLIT (steps of one token per request, at most 16 heads per key head): the four wavefronts hold the SAME rows and
+// walk different key tiles, each with its own staging area and no workgroup barrier inside the walk; their partial
+// (maximum, sum, output) triples meet in LDS at the end.  A decoded token's window is thus read four tiles at a time.
 constexpr int MA_KEYS = 64, MA_VST = MA_KEYS + 8, MA_PST = MA_KEYS + 8;
 
-template <int KS, int CT>
+constexpr size_t ma_stage_bytes(int ks, int ct) {     // one staging area: K tile, transposed V tile
+  return ((size_t)MA_KEYS * (ks * 32 + 8) + (size_t)ct * 16 * MA_VST) * 2;
+}
+constexpr size_t ma_lds_bytes(int ks, int ct, bool split) {
+  return split ? 4 * (ma_stage_bytes(ks, ct) + 16 * MA_PST * 2) : ma_stage_bytes(ks, ct) + 4 * 16 * MA_PST * 2;
+}
+
+template <int KS, int CT, bool SPLIT>
 __global__ __launch_bounds__(256) void window_attn_mfma_kernel(WAttnArgs p) {
   constexpr int DK = KS * 32, KST = DK + 8, DVP = CT * 16;
+  constexpr int STAGE = (int)(ma_stage_bytes(KS, CT) / 2);                 // bf16 elements of one staging area
   extern __shared__ u32x4 lds_raw[];
-  bf16_t* sK = reinterpret_cast<bf16_t*>(lds_raw);          // [64][KST]
-  bf16_t* sVt = sK + MA_KEYS * KST;                          // [DVP][MA_VST]
-  bf16_t* sP = sVt + DVP * MA_VST;                           // [4][16][MA_PST]
-  __shared__ int64_t sRow[MA_KEYS];
+  __shared__ int64_t sRowAll[SPLIT ? 4 : 1][MA_KEYS];
   const int R = p.H / p.G, d = p.d, dv = p.dv;
   const int g = blockIdx.y;
   const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
   const int lc = lane & 15, lg = lane >> 4;
+  bf16_t* base = reinterpret_cast<bf16_t*>(lds_raw);
+  bf16_t* sK = base + (SPLIT ? wv * STAGE : 0);              // [64][KST]
+  bf16_t* sVt = sK + MA_KEYS * KST;                          // [DVP][MA_VST]
+  bf16_t* sPw = base + (SPLIT ? 4 : 1) * STAGE + wv * 16 * MA_PST;   // [16][MA_PST] of this wavefront
+  int64_t* sRow = sRowAll[SPLIT ? wv : 0];
+  constexpr int ST = SPLIT ? 64 : 256;                                    // threads that stage a tile together
+  constexpr int NKC = MA_KEYS * (DK / 8) / ST, NVC = MA_KEYS * (DVP / 8) / ST;   // 16-byte pieces per thread
+  const int stid = SPLIT ? lane : tid;
+  const int row0 = SPLIT ? 0 : wv * 16;                                   // first query row of this wavefront
+  auto sync = [&]() {
+    if constexpr (SPLIT) {      // the area is private to this wavefront: its own LDS accesses complete in order
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    } else {
+      __syncthreads();
+    }
+  };
   const int64_t t_begin = (int64_t)blockIdx.x * p.TQ;
   const int64_t t_end = min(p.tokens, t_begin + p.TQ);
   const bf16_t* cache = reinterpret_cast<const bf16_t*>(p.cache);
   const int cw = p.G * (d + dv);
   bf16_t* out = reinterpret_cast<bf16_t*>(p.out);
-  bf16_t* sPw = sP + wv * 16 * MA_PST;
 
   for (int64_t ts = t_begin; ts < t_end;) {
     const int b = p.seq_of[ts];
@@ -212,11 +238,11 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(WAttnArgs p) {
     const int nq = (int)(te - ts), rows = nq * R;
     const int p0 = p.past[b] + (int)(ts - p.cu_q[b]);
     const int32_t* table = p.tables + (int64_t)b * p.table_cols;
-    const bool wave_on = wv * 16 < rows;
+    const bool wave_on = row0 < rows;
     // query fragments of this wavefront's 16 rows (A operand: lane holds row lc, features 8 lg .. 8 lg + 7 of each step)
     bf16x8 qf[KS];
     {
-      const int rr = wv * 16 + lc;
+      const int rr = row0 + lc;
       const bool ok = rr < rows;
       const float* qrow = ok ? p.q + ((ts + rr / R) * p.H + g * R + rr % R) * d : nullptr;
 #pragma unroll
@@ -234,7 +260,7 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(WAttnArgs p) {
     bool valid[4];
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      const int rr = wv * 16 + lg * 4 + r;
+      const int rr = row0 + lg * 4 + r;
       valid[r] = rr < rows;
       pos[r] = p0 + rr / R;
       slope[r] = exp2f(-8.0f * (float)(g * R + rr % R + 1) / (float)p.H);
@@ -244,35 +270,48 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(WAttnArgs p) {
     f32x4 acc_o[CT];
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct) acc_o[ct] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-    const int wpos_lo = p0 + (wv * 16) / R, wpos_hi = p0 + min(rows - 1, wv * 16 + 15) / R;
+    const int wpos_lo = p0 + row0 / R, wpos_hi = p0 + min(rows - 1, row0 + 15) / R;
 
     const int lo = p.window > 0 ? max(0, p0 - p.window + 1) : 0, hi = p0 + nq - 1;
-    for (int j0 = lo; j0 <= hi; j0 += MA_KEYS) {
-      if (tid < MA_KEYS) {
-        const int kp = j0 + tid;
-        sRow[tid] = kp <= hi ? (int64_t)table[kp / p.block_size] * p.block_size + kp % p.block_size : -1;
+    for (int j0 = lo + (SPLIT ? wv * MA_KEYS : 0); j0 <= hi; j0 += SPLIT ? 4 * MA_KEYS : MA_KEYS) {
+      if (stid < MA_KEYS) {
+        const int kp = j0 + stid;
+        sRow[stid] = kp <= hi ? (int64_t)table[kp / p.block_size] * p.block_size + kp % p.block_size : -1;
       }
-      __syncthreads();
-      for (int c = tid; c < MA_KEYS * (DK / 8); c += 256) {
-        const int key = c / (DK / 8), part = c % (DK / 8);
+      sync();
+      // all of a thread's loads are issued before the first LDS store: one round trip to memory per tile
+      u32x4 kreg[NKC], vreg[NVC];
+#pragma unroll
+      for (int i = 0; i < NKC; ++i) {
+        const int c = stid + i * ST, key = c / (DK / 8), part = c % (DK / 8);
         const int64_t row = sRow[key];
-        u32x4 val = u32x4{0u, 0u, 0u, 0u};
-        if (row >= 0 && part * 8 < d) val = *reinterpret_cast<const u32x4*>(cache + row * cw + g * d + part * 8);
-        *reinterpret_cast<u32x4*>(sK + key * KST + part * 8) = val;
+        kreg[i] = u32x4{0u, 0u, 0u, 0u};
+        if (row >= 0 && part * 8 < d) kreg[i] = *reinterpret_cast<const u32x4*>(cache + row * cw + g * d + part * 8);
       }
-      for (int c = tid; c < MA_KEYS * (DVP / 8); c += 256) {
-        const int key = c % MA_KEYS, part = c / MA_KEYS;
+#pragma unroll
+      for (int i = 0; i < NVC; ++i) {
+        const int c = stid + i * ST, key = c % MA_KEYS, part = c / MA_KEYS;
         const int64_t row = sRow[key];
-        u32x4 val = u32x4{0u, 0u, 0u, 0u};
-        if (row >= 0 && part * 8 < dv) val = *reinterpret_cast<const u32x4*>(cache + row * cw + p.G * d + g * dv + part * 8);
+        vreg[i] = u32x4{0u, 0u, 0u, 0u};
+        if (row >= 0 && part * 8 < dv)
+          vreg[i] = *reinterpret_cast<const u32x4*>(cache + row * cw + p.G * d + g * dv + part * 8);
+      }
+#pragma unroll
+      for (int i = 0; i < NKC; ++i) {
+        const int c = stid + i * ST, key = c / (DK / 8), part = c % (DK / 8);
+        *reinterpret_cast<u32x4*>(sK + key * KST + part * 8) = kreg[i];
+      }
+#pragma unroll
+      for (int i = 0; i < NVC; ++i) {
+        const int c = stid + i * ST, key = c % MA_KEYS, part = c / MA_KEYS;
         uint16_t* dst = reinterpret_cast<uint16_t*>(sVt) + (part * 8) * MA_VST + key;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          dst[(2 * i) * MA_VST] = (uint16_t)(val[i] & 0xffffu);
-          dst[(2 * i + 1) * MA_VST] = (uint16_t)(val[i] >> 16);
+        for (int w = 0; w < 4; ++w) {
+          dst[(2 * w) * MA_VST] = (uint16_t)(vreg[i][w] & 0xffffu);
+          dst[(2 * w + 1) * MA_VST] = (uint16_t)(vreg[i][w] >> 16);
         }
       }
-      __syncthreads();
+      sync();
       // keys this wavefront's rows can see: [wpos_lo - window + 1, wpos_hi]
       const bool need = wave_on && j0 <= wpos_hi && (p.window <= 0 || j0 + MA_KEYS - 1 > wpos_lo - p.window);
       if (need) {
@@ -337,12 +376,46 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(WAttnArgs p) {
           }
         }
       }
-      __syncthreads();
+      sync();
     }
-    if (wave_on) {
+    if constexpr (SPLIT) {
+      // partial results of the four wavefronts: rows of DVP outputs, the maximum and the sum, in each one's V area
+      constexpr int PW = DVP + 2;
+      float* part = reinterpret_cast<float*>(sVt);
+      static_assert((size_t)16 * PW * 4 <= (size_t)DVP * MA_VST * 2, "partials fit the V area");
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        const int rr = wv * 16 + lg * 4 + r;
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) part[(lg * 4 + r) * PW + ct * 16 + lc] = acc_o[ct][r];
+        if (lc == 0) {
+          part[(lg * 4 + r) * PW + DVP] = m_run[r];
+          part[(lg * 4 + r) * PW + DVP + 1] = l_run[r];
+        }
+      }
+      __syncthreads();
+      for (int idx = tid; idx < 16 * DVP; idx += 256) {
+        const int rr = idx / DVP, e = idx % DVP;
+        if (rr >= rows || e >= dv) continue;
+        float m = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < 4; ++w)
+          m = fmaxf(m, reinterpret_cast<const float*>(base + w * STAGE + MA_KEYS * KST)[rr * PW + DVP]);
+        float l = 0.0f, o = 0.0f;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          const float* pw = reinterpret_cast<const float*>(base + w * STAGE + MA_KEYS * KST);
+          const float mw = pw[rr * PW + DVP];
+          const float f = mw == -INFINITY ? 0.0f : __expf(mw - m);
+          l += pw[rr * PW + DVP + 1] * f;
+          o += pw[rr * PW + e] * f;
+        }
+        out[(ts + rr / R) * p.out_rs + (g * R + rr % R) * dv + e] = (bf16_t)(o * p.out_scale / l);
+      }
+      __syncthreads();
+    } else if (wave_on) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int rr = row0 + lg * 4 + r;
         if (!valid[r]) continue;
         const float f = p.out_scale / l_run[r];
         bf16_t* orow = out + (ts + rr / R) * p.out_rs + (g * R + rr % R) * dv;
@@ -357,16 +430,36 @@ __global__ __launch_bounds__(256) void window_attn_mfma_kernel(WAttnArgs p) {
   }
 }
 
-template <int KS>
-hipError_t launch_window_mfma(const WAttnArgs& p, int ct, dim3 grid, hipStream_t s) {
-  const size_t lds = ((size_t)MA_KEYS * (KS * 32 + 8) + (size_t)ct * 16 * MA_VST + 4 * 16 * MA_PST) * sizeof(bf16_t);
-  switch (ct) {
-    case 2: window_attn_mfma_kernel<KS, 2><<<grid, dim3(256), lds, s>>>(p); break;
-    case 4: window_attn_mfma_kernel<KS, 4><<<grid, dim3(256), lds, s>>>(p); break;
-    case 8: window_attn_mfma_kernel<KS, 8><<<grid, dim3(256), lds, s>>>(p); break;
-    default: window_attn_mfma_kernel<KS, 16><<<grid, dim3(256), lds, s>>>(p); break;
+template <int KS, int CT, bool SPLIT>
+hipError_t launch_window_mfma3(const WAttnArgs& p, dim3 grid, hipStream_t s) {
+  constexpr size_t lds = ma_lds_bytes(KS, CT, SPLIT);
+  static size_t allowed = 64 * 1024;
+  if (lds > allowed) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&window_attn_mfma_kernel<KS, CT, SPLIT>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return e;
+    allowed = lds;
   }
+  window_attn_mfma_kernel<KS, CT, SPLIT><<<grid, dim3(256), lds, s>>>(p);
   return hipGetLastError();
+}
+
+template <int KS, int CT>
+hipError_t launch_window_mfma2(const WAttnArgs& p, bool split, dim3 grid, hipStream_t s) {
+  if constexpr (ma_lds_bytes(KS, CT, true) <= 156 * 1024) {
+    if (split) return launch_window_mfma3<KS, CT, true>(p, grid, s);
+  }
+  return launch_window_mfma3<KS, CT, false>(p, grid, s);
+}
+
+template <int KS>
+hipError_t launch_window_mfma(const WAttnArgs& p, int ct, bool split, dim3 grid, hipStream_t s) {
+  switch (ct) {
+    case 2: return launch_window_mfma2<KS, 2>(p, split, grid, s);
+    case 4: return launch_window_mfma2<KS, 4>(p, split, grid, s);
+    case 8: return launch_window_mfma2<KS, 8>(p, split, grid, s);
+    default: return launch_window_mfma2<KS, 16>(p, split, grid, s);
+  }
 }
 
 }  // namespace
@@ -403,15 +496,16 @@ extern "C" int nv_window_attn(const float* q, const void* cache, const int32_t* 
       (uintptr_t)cache % 16 == 0 && getenv("NV_WINDOW_ATTN_MFMA_OFF") == nullptr) {
     const int ks = dim <= 64 ? 2 : dim <= 128 ? 4 : 8;
     const int ct = vdim <= 32 ? 2 : vdim <= 64 ? 4 : vdim <= 128 ? 8 : 16;
-    const size_t lds = ((size_t)MA_KEYS * (ks * 32 + 8) + (size_t)ct * 16 * MA_VST + 4 * 16 * MA_PST) * 2;
-    if (lds <= 64 * 1024) {
+    if (ma_lds_bytes(ks, ct, false) <= 160 * 1024) {
+      const bool split = max_q <= 1 && R <= 16;           // one token per request: the wavefronts split the window
       const int TQm = max_q <= 1 ? 1 : 64 / R;
       WAttnArgs pm{q, cache, block_tables, table_cols, cu_q, past_lens, seq_of_token, out, out_row_stride, tokens, heads,
                    kv_heads, dim, vdim, block_size, window, TQm, MA_KEYS, softcap, out_scale};
       dim3 gridm((unsigned)((tokens + TQm - 1) / TQm), (unsigned)kv_heads);
       hipStream_t st = (hipStream_t)stream;
-      const hipError_t e = ks == 2 ? launch_window_mfma<2>(pm, ct, gridm, st)
-                           : ks == 4 ? launch_window_mfma<4>(pm, ct, gridm, st) : launch_window_mfma<8>(pm, ct, gridm, st);
+      const hipError_t e = ks == 2 ? launch_window_mfma<2>(pm, ct, split, gridm, st)
+                           : ks == 4 ? launch_window_mfma<4>(pm, ct, split, gridm, st)
+                                     : launch_window_mfma<8>(pm, ct, split, gridm, st);
       if (e != hipSuccess) {
         nv_set_error("nv_window_attn: %s", hipGetErrorString(e));
         return NV_ERR_LAUNCH;

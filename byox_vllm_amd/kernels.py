@@ -777,9 +777,10 @@ def rglru_scan(u, gates, y, lam, state, cu_q, past_lens, state_slots, block_widt
     return out
 
 
-def ssd_scan(xbc, z, dt, dt_bias, A_log, D, state, cu_q, past_lens, state_slots, heads, groups, state_size, vdim):
+def ssd_scan(xbc, z, dt, dt_bias, A_log, D, state, cu_q, past_lens, state_slots, heads, groups, state_size, vdim, max_q=1):
     """Selective state-space recurrence over fp32 rows xbc [T, heads*vdim + 2*groups*state] -> fp32 [T, heads*vdim]
-    (already multiplied by silu(z)); ``state`` fp32 [slots, heads, state, vdim]."""
+    (already multiplied by silu(z)); ``state`` fp32 [slots, heads, state, vdim].  ``max_q`` bounds the tokens one
+    request brings (long prompts are walked in parallel runs through a workspace)."""
     require_gpu(xbc, "ssd_scan")
     T = xbc.size(0)
     inner = heads * vdim
@@ -790,7 +791,11 @@ def ssd_scan(xbc, z, dt, dt_bias, A_log, D, state, cu_q, past_lens, state_slots,
     assert dt_bias.dtype == A_log.dtype == D.dtype
     assert cu_q.dtype == past_lens.dtype == state_slots.dtype == torch.int32
     out = torch.empty(T, inner, dtype=torch.float32, device=xbc.device)
+    B = past_lens.numel()
+    nbytes = lib().nv_ssd_scan_workspace_bytes(B, heads, state_size, vdim, max_q)
+    ws = workspace(nbytes, xbc.device, "ssd_scan") if nbytes else None
     check(lib().nv_ssd_scan(ptr(xbc), xbc.stride(0), ptr(z), z.stride(0), ptr(dt), dt.stride(0), ptr(dt_bias), ptr(A_log),
-                            ptr(D), ptr(state), ptr(cu_q), ptr(past_lens), ptr(state_slots), ptr(out), past_lens.numel(),
-                            heads, groups, state_size, vdim, _code32(dt_bias.dtype), stream()), "nv_ssd_scan")
+                            ptr(D), ptr(state), ptr(cu_q), ptr(past_lens), ptr(state_slots), ptr(out), B,
+                            heads, groups, state_size, vdim, max_q, ptr(ws), nbytes, _code32(dt_bias.dtype), stream()),
+          "nv_ssd_scan")
     return out

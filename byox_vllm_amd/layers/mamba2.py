@@ -46,6 +46,6 @@ class Mamba2Mixer(nn.Module):
         xbc, _ = self.conv(proj[:, inner:2 * inner + 2 * gn])
         y = kernels.ssd_scan(xbc, proj[:, :inner], proj[:, 2 * inner + 2 * gn:], self.dt_bias.data, self.A_log.data,
                              self.D.data, self.state, ctx.cu_seqlens_q, ctx.past_lens, ctx.state_slots, self.heads,
-                             self.groups, self.n, self.vdim)
+                             self.groups, self.n, self.vdim, max_q=ctx.max_seqlen_q)
         y = kernels.group_rms_norm_f32(y, self.norm.data, self.norm_groups, self.eps)
         return self.o(y, out_dtype=torch.float32)

@@ -451,7 +451,11 @@ int nv_rglru_scan(const float* u, int64_t u_row_stride, const float* gates, int6
 int nv_ssd_scan(const float* xbc, int64_t xbc_row_stride, const float* z, int64_t z_row_stride, const float* dt,
                 int64_t dt_row_stride, const void* dt_bias, const void* A_log, const void* D, float* state,
                 const int32_t* cu_q, const int32_t* past_lens, const int32_t* state_slots, float* out, int num_seqs,
-                int heads, int groups, int state_size, int vdim, int dtype, nv_stream_t stream);
+                int heads, int groups, int state_size, int vdim, int max_q, void* workspace, size_t workspace_bytes,
+                int dtype, nv_stream_t stream);
+/* Bytes nv_ssd_scan needs when no request brings more than max_q tokens (0 for short steps: long prompts are cut into
+ * runs that are walked side by side, and the runs' end states pass through the workspace). */
+size_t nv_ssd_scan_workspace_bytes(int num_seqs, int heads, int state_size, int vdim, int max_q);
 
 #ifdef __cplusplus
 }

@@ -259,6 +259,35 @@ def test_state_space_scan_in_pieces(H, G, P, N, pieces):
     _close(got, want, 2e-5)
 
 
+@pytest.mark.parametrize("pieces", [[700], [300, 400], [257, 3, 440], [40, 660]])
+def test_state_space_scan_long_prompts_are_walked_in_parallel_runs(pieces):
+    """From 256 tokens per request on, a prompt is cut into runs whose end states meet through a workspace: same
+    numbers as the plain walk, whatever the cut, also beside a short request in the same launch."""
+    from byox_vllm_amd import kernels
+    H, G, P, N = 3, 1, 16, 24
+    xbc, z, dt, dt_bias, A_log, D = _ssd_inputs(700, H, G, P, N, 5)
+    short = _ssd_inputs(5, H, G, P, N, 6)[:3]
+    want = _ssd_plain(xbc, z, dt, dt_bias, A_log, D, H, G, P, N)
+    want_short = _ssd_plain(*short, dt_bias, A_log, D, H, G, P, N)
+    state = torch.full((3, H, N, P), 3.0, device=DEV)
+    params = [t.to(DEV) for t in (dt_bias, A_log, D)]
+    got, at = [], 0
+    for k, n in enumerate(pieces):
+        rows = [xbc[at:at + n], z[at:at + n], dt[at:at + n]]
+        beside = k == 0                                   # the short request rides along in the first step
+        if beside:
+            rows = [torch.cat([s_, r]) for s_, r in zip(short, rows)]
+        cu = _i32([0, 5, 5 + n] if beside else [0, n])
+        out = kernels.ssd_scan(*[r.to(DEV) for r in rows], *params, state, cu, _i32([0, at] if beside else [at]),
+                               _i32([2, 1] if beside else [1]), H, G, N, P, max_q=n)
+        if beside:
+            _close(out[:5], want_short, 2e-5)
+            out = out[5:]
+        got.append(out)
+        at += n
+    _close(torch.cat(got), want, 5e-5)
+
+
 def test_state_space_scan_batch_and_reused_slot():
     """Two requests side by side, then a third one in the slot the first has left: it must start from zero."""
     from byox_vllm_amd import kernels
