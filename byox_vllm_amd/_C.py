@@ -72,6 +72,7 @@ _PROTOS = {
     "nv_dyt_norm": (_i, [_p, _p, _i64, _p, _p, _p, _p, _p, _i64, _i, _i, _p]),
     "nv_rmsnorm_f32": (_i, [_p, _i64, _p, _p, _i64, _i64, _i, _f, _i, _p]),
     "nv_act_mul_f32": (_i, [_p, _p, _i64, _i, _i, _i, _p]),
+    "nv_act_f32": (_i, [_p, _p, _i64, _i, _p, _f, _i, _p]),
     "nv_sample_f32": (_i, [_p, _i64, _p, _p, _i, _i, _u64, _p]),
     "nv_gla_recurrent": (_i, [_p, _i64, _i, _i, _i, _i, _p, _i64, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _f, _f, _f, _i, _p]),
     "nv_latent_kv_store": (_i, [_p, _i64, _p, _p, _p, _f, _p, _p, _i64, _i, _i, _i, _f, _i, _p]),
@@ -84,10 +85,10 @@ _PROTOS = {
     "nv_hc_norm": (_i, [_p, _i, _i, _p, _i64, _p, _p, _p, _i, _f, _p, _p, _i64, _i, _i64, _i, _p]),
     "nv_token_shift": (_i, [_p, _p, _p, _p, _p, _p, _p, _p, _i64, _i, _i, _p]),
     "nv_group_rmsnorm_f32": (_i, [_p, _i64, _p, _p, _i64, _i64, _i, _i, _f, _i, _p]),
-    "nv_qk_norm_store": (_i, [_p, _i64, _i, _i, _i, _p, _p, _p, _f, _f, _p, _p, _p, _i64, _i, _i, _i, _i, _i, _p]),
+    "nv_qk_norm_store": (_i, [_p, _p, _i64, _i, _i, _i, _p, _p, _p, _f, _f, _p, _p, _p, _i64, _i, _i, _i, _i, _i, _p]),
     "nv_window_attn": (_i, [_p, _p, _p, _i, _p, _p, _p, _p, _i64, _i64, _i, _i, _i, _i, _i, _i, _i, _f, _f, _i, _p]),
-    "nv_causal_conv": (_i, [_p, _i64, _p, _p, _p, _p, _p, _p, _p, _p, _i64, _p, _i64, _i64, _i, _i, _i, _i, _p]),
-    "nv_rglru_scan": (_i, [_p, _i64, _p, _i64, _p, _i64, _p, _p, _p, _p, _p, _p, _i64, _i, _i, _i, _f, _f, _i, _p]),
+    "nv_causal_conv": (_i, [_p, _p, _i64, _p, _p, _p, _p, _p, _p, _p, _p, _i64, _p, _i64, _i64, _i, _i, _i, _i, _p]),
+    "nv_rglru_scan": (_i, [_p, _i64, _p, _i64, _p, _p, _i64, _p, _p, _p, _p, _p, _p, _i64, _i, _i, _i, _f, _f, _i, _p]),
     "nv_ssd_scan": (_i, [_p, _i64, _p, _i64, _p, _i64, _p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _p, _sz, _i,
                          _p]),
     "nv_ssd_scan_workspace_bytes": (_sz, [_i, _i, _i, _i, _i]),

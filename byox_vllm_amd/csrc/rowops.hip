@@ -63,6 +63,24 @@ __global__ __launch_bounds__(256) void act_mul_f32_kernel(const float* __restric
   }
 }
 
+// out = f(y): the element-wise epilogue of nv_linear applied to a plain product's fp32 result (same function codes)
+template <typename T>
+__global__ __launch_bounds__(256) void act_f32_kernel(const float* __restrict__ y, T* __restrict__ out, int64_t total,
+                                                      int act, const float* __restrict__ prm, float c) {
+  const float a = act == 2 ? prm[0] : 0.0f, b = act == 2 ? prm[1] : 0.0f;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
+    const float v = y[i];
+    float r;
+    switch (act) {
+      case 0: r = silu_f32(v); break;
+      case 1: r = gelu_tanh_f32(v); break;
+      case 2: r = v > 0.0f ? a * v * v + 0.5f * v : b * (expm1f(v) - v) + 0.5f * v; break;
+      default: r = v * c; break;
+    }
+    st_f32<T>(out + i, r);
+  }
+}
+
 // Gumbel-max sampling from fp32 logits: argmax_j (l_j / T + g_j) with g_j = -log(-log(u_j)), u_j a hash of (seed, row,
 // column); temperature 0 takes the plain argmax.  Ties go to the lowest index.
 __device__ __forceinline__ uint32_t mix32(uint64_t x) {
@@ -136,6 +154,20 @@ extern "C" int nv_act_mul_f32(const float* y, void* out, int64_t rows, int n, in
   if (blocks > 8192) blocks = 8192;
   NV_DISPATCH_T(dtype, act_mul_f32_kernel<T><<<dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream>>>(
                            y, (T*)out, total, n, act));
+  NV_CHECK_LAUNCH();
+  return NV_OK;
+}
+
+extern "C" int nv_act_f32(const float* y, void* out, int64_t total, int act, const float* params, float c, int dtype,
+                          nv_stream_t stream) {
+  NV_CHECK_ARG(y && out, "nv_act_f32: null pointer");
+  NV_CHECK_ARG(dtype == NV_BF16 || dtype == NV_F32, "nv_act_f32: bad dtype %d", dtype);
+  NV_CHECK_ARG(total >= 0 && act >= 0 && act <= 3 && (act != 2 || params), "nv_act_f32: bad shape or activation");
+  if (total == 0) return NV_OK;
+  int64_t blocks = (total + 255) / 256;
+  if (blocks > 16384) blocks = 16384;
+  NV_DISPATCH_T(dtype, act_f32_kernel<T><<<dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream>>>(
+                           y, (T*)out, total, act, params, c));
   NV_CHECK_LAUNCH();
   return NV_OK;
 }

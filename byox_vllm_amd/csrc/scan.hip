@@ -17,7 +17,8 @@ constexpr int CONV_MAX_TAPS = 8;
 __device__ __forceinline__ float softplus_f32(float z) { return fmaxf(z, 0.0f) + log1pf(expf(-fabsf(z))); }
 
 struct ConvArgs {
-  const float* x;         // [tokens, x_rs] inputs (fp32 projections, bias included)
+  const float* x;         // [tokens, x_rs] inputs (fp32 projections)
+  const void* x_bias;     // [C] added to every input before anything else (the slot keeps inputs with it), or null
   int64_t x_rs;
   const void* w;          // [C, taps]
   const void* bias;       // [C] or null
@@ -47,6 +48,7 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(ConvArgs p) {
   if (k > 0 && k < keep) return;
   const T* w = reinterpret_cast<const T*>(p.w) + (int64_t)c * taps;
   const float bias = p.bias ? ld_f32<T>(reinterpret_cast<const T*>(p.bias) + c) : 0.0f;
+  const float xb = p.x_bias ? ld_f32<T>(reinterpret_cast<const T*>(p.x_bias) + c) : 0.0f;
   float wt[CONV_MAX_TAPS];
 #pragma unroll
   for (int j = 0; j < CONV_MAX_TAPS; ++j) wt[j] = j < taps ? ld_f32<T>(w + j) : 0.0f;
@@ -59,7 +61,7 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(ConvArgs p) {
     float v = bias;
 #pragma unroll
     for (int j = 0; j < CONV_MAX_TAPS; ++j)
-      if (j < taps) v += wt[j] * p.x[(t - (keep - j)) * p.x_rs + c];
+      if (j < taps) v += wt[j] * (p.x[(t - (keep - j)) * p.x_rs + c] + xb);
     emit(t, v);
     return;
   }
@@ -77,7 +79,7 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(ConvArgs p) {
     for (int j = 0; j < CONV_MAX_TAPS; ++j) {
       if (j >= taps) continue;
       const int src = kk - (keep - j);
-      v += wt[j] * (src >= 0 ? p.x[(t0 + src) * p.x_rs + c] : st[kk + j]);
+      v += wt[j] * (src >= 0 ? p.x[(t0 + src) * p.x_rs + c] + xb : st[kk + j]);
     }
     emit(t0 + kk, v);
   }
@@ -85,7 +87,7 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(ConvArgs p) {
   for (int i = 0; i < CONV_MAX_TAPS; ++i) {
     if (i >= keep) continue;
     const int src = n - keep + i;
-    slot[(int64_t)i * p.C + c] = src >= 0 ? p.x[(t0 + src) * p.x_rs + c] : st[i + n];
+    slot[(int64_t)i * p.C + c] = src >= 0 ? p.x[(t0 + src) * p.x_rs + c] + xb : st[i + n];
   }
 }
 
@@ -95,6 +97,7 @@ struct RglruArgs {
   const float* gates;     // [tokens, g_rs]: per block of bw channels, bw recurrence-gate logits then bw input-gate logits
   int64_t g_rs;
   const float* y;         // [tokens, y_rs] the other branch before its activation
+  const void* y_bias;     // [C] added to y first, or null
   int64_t y_rs;
   const void* lam;        // [C]
   float* state;           // [slots, C]
@@ -126,6 +129,7 @@ __global__ __launch_bounds__(RG_CHUNKS * RG_CH) void rglru_scan_kernel(RglruArgs
   const int64_t c0 = min((int64_t)t1, (int64_t)t0 + (int64_t)j * len), c1 = min((int64_t)t1, c0 + len);
   const float sp = on ? p.c * softplus_f32(ld_f32<T>(reinterpret_cast<const T*>(p.lam) + ch)) : 0.0f;
   const int gcol = on ? (ch / p.bw) * 2 * p.bw + ch % p.bw : 0;
+  const float yb = (on && p.y_bias) ? ld_f32<T>(reinterpret_cast<const T*>(p.y_bias) + ch) : 0.0f;
   auto step = [&](int64_t t, float& a, float& inp) {
     const float gr = p.gates[t * p.g_rs + gcol], gi = p.gates[t * p.g_rs + gcol + p.bw];
     const float log_a = -sp * sigmoid_f32(gr);
@@ -155,7 +159,7 @@ __global__ __launch_bounds__(RG_CHUNKS * RG_CH) void rglru_scan_kernel(RglruArgs
     float a, inp;
     step(t, a, inp);
     S = a * S + inp;
-    st_f32<T>(out + t * p.out_rs + ch, S * gelu_tanh_f32(p.y[t * p.y_rs + ch]) * p.out_scale);
+    st_f32<T>(out + t * p.out_rs + ch, S * gelu_tanh_f32(p.y[t * p.y_rs + ch] + yb) * p.out_scale);
   }
   if (c1 == t1 && c1 > c0) *slot = S;      // the run that holds the step's last token
 }
@@ -318,7 +322,7 @@ __global__ __launch_bounds__(1024) void ssd_scan_kernel(SsdArgs p, int tc) {
 
 }  // namespace
 
-extern "C" int nv_causal_conv(const float* x, int64_t x_row_stride, const void* w, const void* bias, float* state,
+extern "C" int nv_causal_conv(const float* x, const void* x_bias, int64_t x_row_stride, const void* w, const void* bias, float* state,
                               const int32_t* cu_q, const int32_t* past_lens, const int32_t* state_slots,
                               const int32_t* seq_of_token, float* out_f32, int64_t out_f32_row_stride, void* out_t,
                               int64_t out_t_row_stride, int64_t tokens, int channels, int taps, int act, int dtype,
@@ -330,7 +334,7 @@ extern "C" int nv_causal_conv(const float* x, int64_t x_row_stride, const void* 
                    (act == 0 || act == 1),
                "nv_causal_conv: bad shape (taps up to %d)", CONV_MAX_TAPS);
   if (tokens == 0) return NV_OK;
-  ConvArgs p{x, x_row_stride, w, bias, state, cu_q, past_lens, state_slots, seq_of_token, out_f32, out_f32_row_stride,
+  ConvArgs p{x, x_bias, x_row_stride, w, bias, state, cu_q, past_lens, state_slots, seq_of_token, out_f32, out_f32_row_stride,
              out_t, out_t_row_stride, channels, taps, act};
   NV_DISPATCH_T(dtype, causal_conv_kernel<T><<<dim3((unsigned)tokens, (unsigned)((channels + 255) / 256)), dim3(256), 0,
                                                (hipStream_t)stream>>>(p));
@@ -339,7 +343,7 @@ extern "C" int nv_causal_conv(const float* x, int64_t x_row_stride, const void* 
 }
 
 extern "C" int nv_rglru_scan(const float* u, int64_t u_row_stride, const float* gates, int64_t gates_row_stride,
-                             const float* y, int64_t y_row_stride, const void* lam, float* state, const int32_t* cu_q,
+                             const float* y, const void* y_bias, int64_t y_row_stride, const void* lam, float* state, const int32_t* cu_q,
                              const int32_t* past_lens, const int32_t* state_slots, void* out, int64_t out_row_stride,
                              int num_seqs, int channels, int block_width, float c, float out_scale, int dtype,
                              nv_stream_t stream) {
@@ -348,7 +352,7 @@ extern "C" int nv_rglru_scan(const float* u, int64_t u_row_stride, const float* 
   NV_CHECK_ARG(num_seqs >= 0 && num_seqs <= 65535 && channels > 0 && block_width > 0 && channels % block_width == 0,
                "nv_rglru_scan: bad shape");
   if (num_seqs == 0) return NV_OK;
-  RglruArgs p{u, u_row_stride, gates, gates_row_stride, y, y_row_stride, lam, state, cu_q, past_lens, state_slots, out,
+  RglruArgs p{u, u_row_stride, gates, gates_row_stride, y, y_bias, y_row_stride, lam, state, cu_q, past_lens, state_slots, out,
               out_row_stride, channels, block_width, c, out_scale};
   NV_DISPATCH_T(dtype, rglru_scan_kernel<T><<<dim3((unsigned)((channels + RG_CH - 1) / RG_CH), (unsigned)num_seqs),
                                               dim3(RG_CH, RG_CHUNKS), 0, (hipStream_t)stream>>>(p));

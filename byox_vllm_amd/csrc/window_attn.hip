@@ -17,7 +17,8 @@
 namespace {
 
 struct QkArgs {
-  const float* proj;      // [tokens, proj_rs]: q | k | v at the given column offsets (fp32 projections, bias included)
+  const float* proj;      // [tokens, proj_rs]: q | k | v at the given column offsets (fp32 projections)
+  const void* bias;       // [proj columns] added to the projections (same column offsets), or null
   int64_t proj_rs;
   int q_off, k_off, v_off;
   const void* qn;         // [d] query norm weight
@@ -41,22 +42,34 @@ __global__ __launch_bounds__(256) void qk_norm_store_kernel(QkArgs p) {
   const T* qn = reinterpret_cast<const T*>(p.qn);
   const T* kn = reinterpret_cast<const T*>(p.kn);
   const T* temp = reinterpret_cast<const T*>(p.temp);
+  const T* bias = reinterpret_cast<const T*>(p.bias);
   for (int v = wv; v < p.H + p.G; v += nw) {
     const bool is_q = v < p.H;
-    const float* src = is_q ? row + p.q_off + v * p.d : row + p.k_off + (v - p.H) * p.d;
+    const int col = is_q ? p.q_off + v * p.d : p.k_off + (v - p.H) * p.d;
+    const float* src = row + col;
     float ss = 0.0f;
-    for (int e = lane; e < p.d; e += 64) ss += src[e] * src[e];
+    for (int e = lane; e < p.d; e += 64) {
+      const float x = src[e] + (bias ? ld_f32<T>(bias + col + e) : 0.0f);
+      ss += x * x;
+    }
     ss = wave_sum(ss);
     const float inv = 1.0f / sqrtf(ss / (float)p.d + p.eps);
     if (is_q) {
       const float f = p.scale * (temp ? ld_f32<T>(temp + v) : 1.0f);
-      for (int e = lane; e < p.d; e += 64) p.q_out[t * p.H * p.d + v * p.d + e] = src[e] * inv * ld_f32<T>(qn + e) * f;
+      for (int e = lane; e < p.d; e += 64) {
+        const float x = src[e] + (bias ? ld_f32<T>(bias + col + e) : 0.0f);
+        p.q_out[t * p.H * p.d + v * p.d + e] = x * inv * ld_f32<T>(qn + e) * f;
+      }
     } else if (crow) {
-      for (int e = lane; e < p.d; e += 64) st_f32<T>(crow + (v - p.H) * p.d + e, src[e] * inv * ld_f32<T>(kn + e));
+      for (int e = lane; e < p.d; e += 64) {
+        const float x = src[e] + (bias ? ld_f32<T>(bias + col + e) : 0.0f);
+        st_f32<T>(crow + (v - p.H) * p.d + e, x * inv * ld_f32<T>(kn + e));
+      }
     }
   }
   if (crow)
-    for (int e = threadIdx.x; e < p.G * p.dv; e += blockDim.x) st_f32<T>(crow + p.G * p.d + e, row[p.v_off + e]);
+    for (int e = threadIdx.x; e < p.G * p.dv; e += blockDim.x)
+      st_f32<T>(crow + p.G * p.d + e, row[p.v_off + e] + (bias ? ld_f32<T>(bias + p.v_off + e) : 0.0f));
 }
 
 struct WAttnArgs {
@@ -464,8 +477,8 @@ hipError_t launch_window_mfma(const WAttnArgs& p, int ct, bool split, dim3 grid,
 
 }  // namespace
 
-extern "C" int nv_qk_norm_store(const float* proj, int64_t proj_row_stride, int q_off, int k_off, int v_off,
-                                const void* q_norm, const void* k_norm, const void* temp, float scale, float eps,
+extern "C" int nv_qk_norm_store(const float* proj, const void* bias, int64_t proj_row_stride, int q_off, int k_off,
+                                int v_off, const void* q_norm, const void* k_norm, const void* temp, float scale, float eps,
                                 const int32_t* slot_mapping, void* cache, float* q_out, int64_t tokens, int heads,
                                 int kv_heads, int dim, int vdim, int dtype, nv_stream_t stream) {
   NV_CHECK_ARG(proj && q_norm && k_norm && slot_mapping && cache && q_out, "nv_qk_norm_store: null pointer");
@@ -473,7 +486,7 @@ extern "C" int nv_qk_norm_store(const float* proj, int64_t proj_row_stride, int 
   NV_CHECK_ARG(tokens >= 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && dim > 0 && vdim > 0,
                "nv_qk_norm_store: bad shape");
   if (tokens == 0) return NV_OK;
-  QkArgs p{proj, proj_row_stride, q_off, k_off, v_off, q_norm, k_norm, temp, slot_mapping, cache, q_out, heads, kv_heads,
+  QkArgs p{proj, bias, proj_row_stride, q_off, k_off, v_off, q_norm, k_norm, temp, slot_mapping, cache, q_out, heads, kv_heads,
            dim, vdim, scale, eps};
   NV_DISPATCH_T(dtype, qk_norm_store_kernel<T><<<dim3((unsigned)tokens), dim3(256), 0, (hipStream_t)stream>>>(p));
   NV_CHECK_LAUNCH();

@@ -459,7 +459,7 @@ def linear(x, w, bias=None, out=None, out_dtype=None, *, rows=None, a_rows=None,
     M = x.size(0) if rows is None else rows
     # prefill-sized plain products of a 16-bit model go where the engine sends its other many-row products: the vendor
     # library, here with the result left in fp32
-    if (epilogue in (EPI_NONE, EPI_GLU) and batch == 1 and group_offsets is None and a_rows is None and bias is None and out is None
+    if (epilogue in (EPI_NONE, EPI_GLU, EPI_ACT) and batch == 1 and group_offsets is None and a_rows is None and bias is None and out is None
             and rows is None and x.dtype == torch.bfloat16 and (out_dtype or x.dtype) in (torch.float32, torch.bfloat16)
             and w.dim() == 2 and w.is_contiguous() and x.stride(0) % 8 == 0 and use_many_rows_path(M, K, n) and K % 8 == 0
             and n % 8 == 0 and x.data_ptr() % 16 == 0):
@@ -467,6 +467,11 @@ def linear(x, w, bias=None, out=None, out_dtype=None, *, rows=None, a_rows=None,
             y = _linear_many_rows(x, w, M, 2 * n, K, torch.float32)
             out = torch.empty(M, n, dtype=out_dtype or x.dtype, device=x.device)
             check(lib().nv_act_mul_f32(ptr(y), ptr(out), M, n, act, _code32(out.dtype), stream()), "nv_act_mul_f32")
+            return out
+        if epilogue == EPI_ACT:      # the element-wise function in one pass over the library's fp32 result
+            y = _linear_many_rows(x, w, M, n, K, torch.float32)
+            out = torch.empty(M, n, dtype=out_dtype or x.dtype, device=x.device)
+            check(lib().nv_act_f32(ptr(y), ptr(out), M * n, act, ptr(gate), cap, _code32(out.dtype), stream()), "nv_act_f32")
             return out
         return _linear_many_rows(x, w, M, n, K, out_dtype or x.dtype)
     grid_rows = M if group_offsets is None else (max_group_rows if max_group_rows is not None else M)
@@ -707,9 +712,11 @@ def group_rms_norm_f32(x, w, groups, eps, out=None):
     return out
 
 
-def qk_norm_store(proj, offsets, q_norm, k_norm, temp, scale, eps, slot_mapping, cache, heads, kv_heads, dim, vdim):
+def qk_norm_store(proj, offsets, q_norm, k_norm, temp, scale, eps, slot_mapping, cache, heads, kv_heads, dim, vdim,
+                  bias=None):
     """fp32 projections [T, *] with q | k | v at ``offsets`` -> fp32 queries [T, heads * dim] (normalised, times scale and
-    the head's temperature); normalised keys and values go to the cache rows [G * dim | G * vdim] of ``slot_mapping``."""
+    the head's temperature); normalised keys and values go to the cache rows [G * dim | G * vdim] of ``slot_mapping``.
+    ``bias`` (a vector over the projection's columns) is added to the projections first."""
     require_gpu(proj, "qk_norm_store")
     T = proj.size(0)
     assert proj.dtype == torch.float32 and proj.stride(1) == 1 and slot_mapping.dtype == torch.int32
@@ -718,8 +725,10 @@ def qk_norm_store(proj, offsets, q_norm, k_norm, temp, scale, eps, slot_mapping,
     assert temp is None or (temp.numel() == heads and temp.dtype == cache.dtype)
     q_off, k_off, v_off = offsets
     assert max(q_off + heads * dim, k_off + kv_heads * dim, v_off + kv_heads * vdim) <= proj.size(1)
+    assert bias is None or (bias.dtype == cache.dtype and bias.is_contiguous() and bias.numel() <= proj.size(1)
+                            and bias.numel() >= max(q_off + heads * dim, k_off + kv_heads * dim, v_off + kv_heads * vdim))
     q = torch.empty(T, heads * dim, dtype=torch.float32, device=proj.device)
-    check(lib().nv_qk_norm_store(ptr(proj), proj.stride(0), q_off, k_off, v_off, ptr(q_norm), ptr(k_norm), ptr(temp),
+    check(lib().nv_qk_norm_store(ptr(proj), ptr(bias), proj.stride(0), q_off, k_off, v_off, ptr(q_norm), ptr(k_norm), ptr(temp),
                                  scale, eps, ptr(slot_mapping), ptr(cache), ptr(q), T, heads, kv_heads, dim, vdim,
                                  _code32(cache.dtype), stream()), "nv_qk_norm_store")
     return q
@@ -742,7 +751,8 @@ def window_attn(q, cache, block_tables, cu_q, past_lens, seq_of_token, max_q, he
     return out
 
 
-def causal_conv(x, w, bias, state, cu_q, past_lens, state_slots, seq_of_token, act=0, want_f32=True, want_t=False):
+def causal_conv(x, w, bias, state, cu_q, past_lens, state_slots, seq_of_token, act=0, want_f32=True, want_t=False,
+                x_bias=None):
     """Per-channel causal convolution of fp32 rows ``x`` [T, C] (a column slice is fine) with ``w`` [C, taps]; ``state``
     fp32 [slots, taps - 1, C].  -> (fp32 result or None, result in w's dtype or None)."""
     require_gpu(x, "causal_conv")
@@ -754,13 +764,15 @@ def causal_conv(x, w, bias, state, cu_q, past_lens, state_slots, seq_of_token, a
     assert cu_q.dtype == past_lens.dtype == state_slots.dtype == seq_of_token.dtype == torch.int32
     of = torch.empty(T, C, dtype=torch.float32, device=x.device) if want_f32 else None
     ot = torch.empty(T, C, dtype=w.dtype, device=x.device) if want_t else None
-    check(lib().nv_causal_conv(ptr(x), x.stride(0), ptr(w), ptr(bias), ptr(state), ptr(cu_q), ptr(past_lens),
+    assert x_bias is None or (x_bias.numel() == C and x_bias.dtype == w.dtype and x_bias.stride(0) == 1)
+    check(lib().nv_causal_conv(ptr(x), ptr(x_bias), x.stride(0), ptr(w), ptr(bias), ptr(state), ptr(cu_q), ptr(past_lens),
                                ptr(state_slots), ptr(seq_of_token), ptr(of), C, ptr(ot), C, T, C, taps, act,
                                _code32(w.dtype), stream()), "nv_causal_conv")
     return of, ot
 
 
-def rglru_scan(u, gates, y, lam, state, cu_q, past_lens, state_slots, block_width, out, c=8.0, out_scale=1.0):
+def rglru_scan(u, gates, y, lam, state, cu_q, past_lens, state_slots, block_width, out, c=8.0, out_scale=1.0,
+               y_bias=None):
     """Real-gated linear recurrence over fp32 rows u [T, C]; ``gates`` fp32 [T, 2C] (per block: recurrence-gate logits,
     then input-gate logits); ``y`` fp32 [T, C] is the other branch before its GELU; ``state`` fp32 [slots, C];
     ``out`` [T, >= C] in lam's dtype."""
@@ -771,7 +783,8 @@ def rglru_scan(u, gates, y, lam, state, cu_q, past_lens, state_slots, block_widt
     assert y.shape == (T, C) and state.is_contiguous() and state.size(-1) == C and lam.numel() == C
     assert out.dtype == lam.dtype and out.size(0) == T and out.size(1) >= C and C % block_width == 0
     assert cu_q.dtype == past_lens.dtype == state_slots.dtype == torch.int32
-    check(lib().nv_rglru_scan(ptr(u), u.stride(0), ptr(gates), gates.stride(0), ptr(y), y.stride(0), ptr(lam), ptr(state),
+    assert y_bias is None or (y_bias.numel() == C and y_bias.dtype == lam.dtype and y_bias.stride(0) == 1)
+    check(lib().nv_rglru_scan(ptr(u), u.stride(0), ptr(gates), gates.stride(0), ptr(y), ptr(y_bias), y.stride(0), ptr(lam), ptr(state),
                               ptr(cu_q), ptr(past_lens), ptr(state_slots), ptr(out), out.stride(0), past_lens.numel(), C,
                               block_width, c, out_scale, _code32(lam.dtype), stream()), "nv_rglru_scan")
     return out

@@ -21,8 +21,9 @@ class CausalConv1d(nn.Module):
     def state_spec(self) -> dict:
         return {"shape": (self.taps - 1, self.channels)}
 
-    def forward(self, x: torch.Tensor, want_f32: bool = True, want_t: bool = False):
-        """``x`` fp32 [T, channels] (a column slice of a wider buffer is fine) -> (fp32 rows, rows in the model dtype)."""
+    def forward(self, x: torch.Tensor, want_f32: bool = True, want_t: bool = False, x_bias: torch.Tensor | None = None):
+        """``x`` fp32 [T, channels] (a column slice of a wider buffer is fine; ``x_bias`` is added to it first)
+        -> (fp32 rows, rows in the model dtype)."""
         ctx = get_context()
         return kernels.causal_conv(x, self.weight.data, self.bias.data, self.state, ctx.cu_seqlens_q, ctx.past_lens,
-                                   ctx.state_slots, ctx.seq_of_token, act=self.act, want_f32=want_f32, want_t=want_t)
+                                   ctx.state_slots, ctx.seq_of_token, act=self.act, want_f32=want_f32, want_t=want_t, x_bias=x_bias)

@@ -43,13 +43,15 @@ class RealGatedLRU(nn.Module):
     def state_modules(self):
         return [self.conv, self]
 
-    def forward(self, x: torch.Tensor, y: torch.Tensor, out: torch.Tensor, out_scale: float = 1.0) -> torch.Tensor:
-        """``x``, ``y`` fp32 [T, channels] (column slices are fine); ``out`` [T, >= channels] in the model dtype."""
+    def forward(self, x: torch.Tensor, y: torch.Tensor, out: torch.Tensor, out_scale: float = 1.0,
+                x_bias: torch.Tensor | None = None, y_bias: torch.Tensor | None = None) -> torch.Tensor:
+        """``x``, ``y`` fp32 [T, channels] (column slices are fine; their biases may still be to add); ``out``
+        [T, >= channels] in the model dtype."""
         ctx = get_context()
-        u32, ut = self.conv(x, want_f32=True, want_t=self.lam.dtype != torch.float32)
+        u32, ut = self.conv(x, want_f32=True, want_t=self.lam.dtype != torch.float32, x_bias=x_bias)
         ut = u32 if ut is None else ut
         bw = self.bw
         g = kernels.linear(ut, self.gates.data, self.gates_bias.data, out_dtype=torch.float32, batch=self.blocks,
                            a_batch_stride=bw, w_batch_stride=2 * bw * bw, out_batch_stride=2 * bw)
         return kernels.rglru_scan(u32, g, y, self.lam.data, self.state, ctx.cu_seqlens_q, ctx.past_lens, ctx.state_slots,
-                                  bw, out, c=self.c, out_scale=out_scale)
+                                  bw, out, c=self.c, out_scale=out_scale, y_bias=y_bias)

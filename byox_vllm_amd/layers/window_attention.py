@@ -36,11 +36,13 @@ class WindowAttention(nn.Module):
     def sizes(self) -> dict:
         return {"q": self.heads * self.dim, "k": self.kv_heads * self.dim, "v": self.kv_heads * self.vdim}
 
-    def forward(self, proj: torch.Tensor, offsets: tuple, out: torch.Tensor, out_scale: float = 1.0) -> torch.Tensor:
-        """``proj`` fp32 [T, *] with q | k | v at ``offsets``; ``out`` [T, >= heads * vdim] in the model dtype."""
+    def forward(self, proj: torch.Tensor, offsets: tuple, out: torch.Tensor, out_scale: float = 1.0,
+                bias: torch.Tensor | None = None) -> torch.Tensor:
+        """``proj`` fp32 [T, *] with q | k | v at ``offsets`` (``bias``, over the same columns, is still to be added);
+        ``out`` [T, >= heads * vdim] in the model dtype."""
         ctx = get_context()
         q = kernels.qk_norm_store(proj, offsets, self.q_norm.data, self.k_norm.data, self.temp.data, self.scale, self.eps,
-                                  ctx.slot_mapping, self.cache, self.heads, self.kv_heads, self.dim, self.vdim)
+                                  ctx.slot_mapping, self.cache, self.heads, self.kv_heads, self.dim, self.vdim, bias=bias)
         return kernels.window_attn(q, self.cache, ctx.block_tables, ctx.cu_seqlens_q, ctx.past_lens, ctx.seq_of_token,
                                    ctx.max_seqlen_q, self.heads, self.kv_heads, self.dim, self.vdim, self.block_size,
                                    self.window, self.softcap, out, out_scale)

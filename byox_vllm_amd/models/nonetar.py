@@ -72,12 +72,15 @@ class ParallelMixer(nn.Module):
         param.data[:, at:at + n].copy_(tensor)
 
     def forward(self, h: torch.Tensor) -> torch.Tensor:
-        proj = self.inp(h, out_dtype=torch.float32)
+        # the biases are added where the projection is consumed: the product needs no epilogue and a prompt's rows go
+        # through the engine's plain many-row route
+        bias = self.inp.bias.data
+        proj = kernels.linear(h, self.inp.weight.data, out_dtype=torch.float32)
         both = torch.empty(h.size(0), self.attn_cols + self.rec_cols, dtype=h.dtype, device=h.device)
-        self.attn(proj, (self.at["q"], self.at["k"], self.at["v"]), both, self.left_scale)
-        c = self.rec_cols
-        self.rec(proj[:, self.at["x"]:self.at["x"] + c], proj[:, self.at["y"]:self.at["y"] + c], both[:, self.attn_cols:],
-                 self.right_scale)
+        self.attn(proj, (self.at["q"], self.at["k"], self.at["v"]), both, self.left_scale, bias=bias)
+        c, ax, ay = self.rec_cols, self.at["x"], self.at["y"]
+        self.rec(proj[:, ax:ax + c], proj[:, ay:ay + c], both[:, self.attn_cols:], self.right_scale,
+                 x_bias=bias[ax:ax + c], y_bias=bias[ay:ay + c])
         return self.o(both, out_dtype=torch.float32)
 
 

@@ -364,6 +364,8 @@ int nv_rmsnorm_f32(const float* x, int64_t x_row_stride, const void* w, void* ou
                    int n, float eps, int dtype, nv_stream_t stream);
 
 /* out[m][j] = act(y[m][j]) * y[m][n + j] over fp32 rows [gate | up] of a plain product; act 0 SiLU, 1 tanh-form GELU. */
+/* nv_act_f32: out = f(y) element-wise over fp32 rows of a plain product, f as in nv_linear's epilogue 4. */
+int nv_act_f32(const float* y, void* out, int64_t total, int act, const float* params, float c, int dtype, nv_stream_t stream);
 int nv_act_mul_f32(const float* y, void* out, int64_t rows, int n, int act, int dtype, nv_stream_t stream);
 
 /* Sampler over fp32 logits: temperature 0 -> argmax (lowest index on ties), else Gumbel-max with noise hashed from
@@ -420,11 +422,14 @@ int nv_group_rmsnorm_f32(const float* x, int64_t x_row_stride, const void* w, vo
                          int64_t rows, int groups, int n, float eps, int dtype, nv_stream_t stream);
 
 /* ---- softmax attention with shaped scores over a paged cache of rows [k: G * dim | v: G * vdim] (csrc/window_attn.hip) ----
- * nv_qk_norm_store: per-head RMS norm of the fp32 q and k projections (weights shared by the heads), q * scale *
+ * nv_qk_norm_store: per-head RMS norm of the fp32 q and k projections plus `bias` (a vector over the projection's columns,
+ *   may be null: a projection's bias can be left to its consumers, so the product itself needs no epilogue; the same
+ *   holds for x_bias of nv_causal_conv and y_bias of nv_rglru_scan); weights shared by the heads, q * scale *
  *   temp[h] left in fp32 [tokens, heads * dim], normalised k and v written to cache row slot_mapping[t] (-1: skipped).
  * nv_window_attn: score = cap(q . k) - 2^(-8 (h + 1) / heads) * (i - j) over keys 0 <= i - j < window (0: all earlier),
  *   cap(z) = softcap * tanh(z / softcap) (softcap 0: none); out[t][h * vdim ..] = out_scale * softmax-weighted values. */
-int nv_qk_norm_store(const float* proj, int64_t proj_row_stride, int q_off, int k_off, int v_off, const void* q_norm,
+int nv_qk_norm_store(const float* proj, const void* bias, int64_t proj_row_stride, int q_off, int k_off, int v_off,
+                     const void* q_norm,
                      const void* k_norm, const void* temp, float scale, float eps, const int32_t* slot_mapping,
                      void* cache, float* q_out, int64_t tokens, int heads, int kv_heads, int dim, int vdim, int dtype,
                      nv_stream_t stream);
@@ -440,12 +445,12 @@ int nv_window_attn(const float* q, const void* cache, const int32_t* block_table
  *   gelu_tanh(y); gates hold, per block of block_width channels, the gr logits followed by the gi logits.
  * nv_ssd_scan: per head, S [state, vdim] <- exp(-exp(A_log) dt) S + dt B x^T, y = S^T C + D x, dt = softplus(raw +
  *   dt_bias), out = y * silu(z) in fp32; xbc rows hold x | B | C with B and C shared by heads / groups heads. */
-int nv_causal_conv(const float* x, int64_t x_row_stride, const void* w, const void* bias, float* state,
+int nv_causal_conv(const float* x, const void* x_bias, int64_t x_row_stride, const void* w, const void* bias, float* state,
                    const int32_t* cu_q, const int32_t* past_lens, const int32_t* state_slots, const int32_t* seq_of_token,
                    float* out_f32, int64_t out_f32_row_stride, void* out_t, int64_t out_t_row_stride, int64_t tokens,
                    int channels, int taps, int act, int dtype, nv_stream_t stream);
 int nv_rglru_scan(const float* u, int64_t u_row_stride, const float* gates, int64_t gates_row_stride, const float* y,
-                  int64_t y_row_stride, const void* lam, float* state, const int32_t* cu_q, const int32_t* past_lens,
+                  const void* y_bias, int64_t y_row_stride, const void* lam, float* state, const int32_t* cu_q, const int32_t* past_lens,
                   const int32_t* state_slots, void* out, int64_t out_row_stride, int num_seqs, int channels,
                   int block_width, float c, float out_scale, int dtype, nv_stream_t stream);
 int nv_ssd_scan(const float* xbc, int64_t xbc_row_stride, const float* z, int64_t z_row_stride, const float* dt,

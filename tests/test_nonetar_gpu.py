@@ -149,15 +149,17 @@ def test_causal_convolution_in_pieces(taps, pieces):
     from byox_vllm_amd import kernels
     torch.manual_seed(taps)
     C = 70
-    x, w, b = torch.randn(30, C + 5), torch.randn(C, taps), torch.randn(C)
-    want = O.silu(O.causal_conv(x[:, 2:2 + C].double(), w.double(), b.double()))
+    x, w, b, xb = torch.randn(30, C + 5), torch.randn(C, taps), torch.randn(C), torch.randn(C)
+    # the inputs' own bias is added by the kernel (the product that made x has no epilogue); the slot keeps x + bias
+    want = O.silu(O.causal_conv(x[:, 2:2 + C].double() + xb.double(), w.double(), b.double()))
     state = torch.full((2, taps - 1, C), 5.0, device=DEV)
     xd = x.to(DEV)
-    got = torch.cat([kernels.causal_conv(xd[a:a + n, 2:2 + C], w.to(DEV), b.to(DEV), state, cu, past, slots, seq_of, act=1)[0]
+    got = torch.cat([kernels.causal_conv(xd[a:a + n, 2:2 + C], w.to(DEV), b.to(DEV), state, cu, past, slots, seq_of, act=1,
+                                         x_bias=xb.to(DEV))[0]
                      for a, n, cu, past, slots, seq_of in _steps(pieces, slot=1)])
     _close(got, want, 1e-5)
     if taps > 1:
-        assert torch.equal(state[1].cpu(), x[30 - (taps - 1):, 2:2 + C])
+        assert torch.equal(state[1].cpu(), x[30 - (taps - 1):, 2:2 + C] + xb)
 
 
 def test_causal_convolution_batch_of_unequal_requests_and_both_outputs():
