@@ -65,6 +65,17 @@ def plain_config():
     ], streams=None, logit_scale=2.0)
 
 
+def ssm_only_config():
+    """No layer owns cache rows: the page pool stays empty-handed while block tables still grow."""
+    return config(50, 40, [(mamba2(2, 1, 8, 16, 4, 2), dense(24)), (mamba2(5, 5, 4, 4, 3, 1), None)], streams=2)
+
+
+def attention_only_config():
+    """Only parallel layers, none with a feed-forward; eight query heads on one key/value head."""
+    return config(90, 64, [(parallel(8, 1, 8, 16, 7, 24, 3, 3), None), (parallel(2, 2, 24, 8, 100, 40, 1, 2, softcap=None), None)],
+                  streams=2, logit_scale=1.5)
+
+
 def aligned_config():
     """Sizes in multiples of 16 and 32, where the 16-bit engine takes its matrix-core kernels; a window of exactly one
     page."""

@@ -6,8 +6,8 @@ import math
 import pytest
 import torch
 
-from nonetar_cases import (aligned_config, engine_config, mixed_config, odd_config, plain_config, random_checkpoint,
-                           row_error, row_errors)
+from nonetar_cases import (aligned_config, attention_only_config, engine_config, mixed_config, odd_config, plain_config,
+                           random_checkpoint, row_error, row_errors, ssm_only_config)
 from oracle import nonetar as O
 
 pytestmark = pytest.mark.gpu
@@ -479,10 +479,12 @@ class Engine:
         return {n: torch.cat(v) for n, v in out.items()}
 
 
-CASES = {"mixed": mixed_config, "odd": odd_config, "plain": plain_config, "aligned": aligned_config}
+CASES = {"mixed": mixed_config, "odd": odd_config, "plain": plain_config, "aligned": aligned_config,
+         "ssm_only": ssm_only_config, "attention_only": attention_only_config}
 
 
-@pytest.fixture(scope="module", params=[(n, dt) for n in CASES for dt in (torch.float32, torch.bfloat16)],
+@pytest.fixture(scope="module", params=[(n, dt) for n in CASES for dt in (torch.float32, torch.bfloat16)
+                                        if dt == torch.float32 or n not in ("ssm_only",)],
                 ids=lambda p: f"{p[0]}-{str(p[1])[6:]}")
 def setup(request):
     name, dtype = request.param

@@ -6,7 +6,8 @@ import json
 import pytest
 import torch
 
-from nonetar_cases import aligned_config, mixed_config, odd_config, plain_config, random_checkpoint
+from nonetar_cases import (aligned_config, attention_only_config, mixed_config, odd_config, plain_config,
+                           random_checkpoint, ssm_only_config)
 from oracle import nonetar as O
 
 F64 = torch.float64
@@ -37,6 +38,15 @@ def test_config_from_a_model_folder(tmp_path):
     c = Config(str(tmp_path), dtype="float32", kvcache_block_size=32, max_num_seqs=3)
     assert c.portioned and c.num_state_slots == 3 and c.hf_config.dtype == torch.float32
     assert c.hf_config.layers[1]["mixer"]["right"]["blocks"] == 3
+
+
+def test_a_model_without_attention_owns_no_pages_and_one_without_state_space_layers_still_has_slots():
+    from byox_vllm_amd.models.nonetar import NonetarForCausalLM, nonetar_config
+    ssm = NonetarForCausalLM(nonetar_config(ssm_only_config(), dtype=torch.float32))
+    assert ssm.page_layers() == [] and len(ssm.state_layers()) == 6
+    att = NonetarForCausalLM(nonetar_config(attention_only_config(), dtype=torch.float32))
+    assert [m.page_spec()["width"] for m in att.page_layers()] == [1 * (8 + 16), 2 * (24 + 8)]
+    assert len(att.state_layers()) == 6
 
 
 @pytest.mark.parametrize("make", [mixed_config, odd_config, plain_config, aligned_config])
