@@ -556,7 +556,7 @@ def test_mixed_batches_reuse_pages_and_slots(setup):
     schedule = [[("a", 30), ("b", 5)], [("a", 1), ("b", 20), ("c", 2)], [("a", 2), ("b", 1)], [("b", 1), ("d", 7), ("a", 1)],
                 [("a", 40), ("d", 1), ("b", 4)], [("d", 30)], [("a", 1), ("d", 1)], [("a", 8), ("d", 11)]]
     _check(setup, setup[5].replay(reqs, schedule))
-    # the same requests again, in slots and pages that the first round has used
+    # the same requests again, in slots and pages that the first pass has used
     _check(setup, setup[5].replay(reqs, [[("d", 50), ("c", 1)], [("c", 1), ("b", 31)], [("a", 83)]]))
 
 
